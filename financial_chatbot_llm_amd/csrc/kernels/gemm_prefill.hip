@@ -203,7 +203,7 @@ __device__ __forceinline__ void read_x(const char* __restrict__ h, FragPair (&b)
 // K-tile past the phase barriers into its last phase (1 + 31 MFMAs between barriers instead of 8
 // per phase), so the partner wave's fragment reads never overlapped them and every fragment was
 // live at once (the balanced schedule then spilled 250 VGPRs).  The bf16 v_mfma_f32_16x16x32
-// stayed in place.  tests/test_vw_asm_hazards.py checks the phase layout of both.
+// stayed in place.
 template <int F0, int T0, bool FP8, bool MXI = false>
 __device__ __forceinline__ void mma(f32x4 (&acc)[8][4], const FragPair (&a)[4], const FragPair (&b)[2],
                                     unsigned sc = 0) {
