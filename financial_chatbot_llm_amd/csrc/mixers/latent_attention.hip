@@ -1,0 +1,241 @@
+// Latent (low-rank key/value) attention over a paged latent cache, with a sliding window.
+//
+// The cache row of a token is [c: R | k_rot: Dr]: the RMS-normed key/value latent and the one
+// rotated key part that all heads share.  Attention runs in the latent space ("absorbed" form):
+// the caller folds each head's key up-projection into its query, q_lat[h] = W_uk[h]^T q_nope[h],
+// so the score of head h for key j is (q_lat[h] . c_j + q_rot[h] . k_rot_j) * scale and the output
+// is o_lat[h] = sum_j p_j c_j; the caller applies the value up-projection to o_lat.  Keys and values
+// of all heads are therefore the same cache rows (one read per key serves every head).
+//
+//   mx_latent_prep    RMS norm of the latent, rotary embedding (interleaved pairs, angle = pos *
+//                     inv_freq[i] in f32) of k_rot and of every head's q_rot, cache write.
+//   mx_latent_attend  windowed causal softmax attention: query at position p sees keys j with
+//                     0 <= p - j < window.  Scores, softmax and accumulation in f32.  The head's
+//                     output is multiplied by sigmoid(gate[t, h]) when a gate is given.
+#include "mx_common.h"
+
+namespace {
+
+constexpr int PAGE = 64;            // tokens per cache page
+
+// one block per token
+template <typename T>
+__global__ void latent_prep_kernel(const T* __restrict__ kv, long skv, const float* __restrict__ norm_w, float eps,
+                                   const float* __restrict__ inv_freq, int rot_dims, const int* __restrict__ pos,
+                                   const int* __restrict__ slots, T* __restrict__ cache, const T* __restrict__ q,
+                                   long sq, int q_head_stride, int q_rot_off, T* __restrict__ q_rot, int H, int R,
+                                   int Dr) {
+  __shared__ float scratch[16];
+  const long t = blockIdx.x;
+  const int slot = slots[t];
+  const float p = (float)pos[t];
+  const T* row = kv + t * skv;
+  const int D = R + Dr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+    const float v = ldf(row + i);
+    ss += v * v;
+  }
+  ss = mx_block_sum(ss, scratch);
+  const float k = 1.0f / sqrtf(ss / (float)R + eps);
+  if (slot >= 0) {
+    T* dst = cache + (long)slot * D;
+    for (int i = threadIdx.x; i < R; i += blockDim.x) stf(dst + i, ldf(row + i) * k * norm_w[i]);
+    for (int i = threadIdx.x; i < Dr / 2; i += blockDim.x) {
+      const float u = ldf(row + R + 2 * i), v = ldf(row + R + 2 * i + 1);
+      if (2 * i + 1 < rot_dims) {
+        float sn, cs;
+        sincosf(p * inv_freq[i], &sn, &cs);
+        stf(dst + R + 2 * i, u * cs - v * sn);
+        stf(dst + R + 2 * i + 1, v * cs + u * sn);
+      } else {
+        stf(dst + R + 2 * i, u);
+        stf(dst + R + 2 * i + 1, v);
+      }
+    }
+    if ((Dr & 1) && threadIdx.x == 0) stf(dst + R + Dr - 1, ldf(row + R + Dr - 1));
+  }
+  // queries: head h's rotated part is q[t][h * q_head_stride + q_rot_off ..+Dr]
+  const int half = Dr / 2;
+  for (int e = threadIdx.x; e < H * half; e += blockDim.x) {
+    const int h = e / half, i = e - h * half;
+    const T* qs = q + t * sq + (long)h * q_head_stride + q_rot_off;
+    T* qd = q_rot + (t * H + h) * Dr;
+    const float u = ldf(qs + 2 * i), v = ldf(qs + 2 * i + 1);
+    if (2 * i + 1 < rot_dims) {
+      float sn, cs;
+      sincosf(p * inv_freq[i], &sn, &cs);
+      stf(qd + 2 * i, u * cs - v * sn);
+      stf(qd + 2 * i + 1, v * cs + u * sn);
+    } else {
+      stf(qd + 2 * i, u);
+      stf(qd + 2 * i + 1, v);
+    }
+  }
+  if (Dr & 1)
+    for (int h = threadIdx.x; h < H; h += blockDim.x)
+      stf(q_rot + (t * H + h) * Dr + Dr - 1, ldf(q + t * sq + (long)h * q_head_stride + q_rot_off + Dr - 1));
+}
+
+// Work layout: a block owns QT consecutive rows of one segment and HB heads; its QT*HB (row, head)
+// items are dealt round-robin to the 4 waves (<= ITEMS per wave).  Key tiles of KT cache rows are
+// staged in LDS once per block and shared by all items.  Per item and tile:
+//   phase 1  lane j scores key j (q read from a per-wave LDS copy: broadcast; the key row stride
+//            is odd in 4-byte words: conflict-free),
+//   phase 2  lane l accumulates value columns l, l+64, ... over the tile's keys.
+constexpr int ATT_WAVES = 4;
+constexpr int ATT_ITEMS = 8;        // items per wave
+constexpr int ATT_RPL = 8;          // value columns per lane: R <= 512
+
+template <typename T>
+__global__ void __launch_bounds__(ATT_WAVES * 64)
+latent_attend_kernel(const T* __restrict__ q_lat, const T* __restrict__ q_rot, const T* __restrict__ cache,
+                     const int* __restrict__ cu, const int* __restrict__ pos, const int* __restrict__ bt, int btw,
+                     const T* __restrict__ gate, long sgate, int window, float scale, T* __restrict__ out,
+                     int H, int R, int Dr, int QT, int HB, int KT, int ldk) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int D = R + Dr;
+  T* ktile = reinterpret_cast<T*>(smem);                                  // [KT][ldk]
+  float* qbuf = reinterpret_cast<float*>(smem + (((size_t)KT * ldk * sizeof(T) + 15) & ~(size_t)15));  // [4][D]
+  float* pbuf = qbuf + ATT_WAVES * D;                                     // [4][64]
+  const int s = blockIdx.z;
+  const int r0 = cu[s], n = cu[s + 1] - r0;
+  const int t0 = blockIdx.x * QT;
+  if (t0 >= n) return;
+  const int nq = min(QT, n - t0);
+  const int h0 = blockIdx.y * HB;
+  const int nh = min(HB, H - h0);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int p_first = pos[r0 + t0], p_last = pos[r0 + t0 + nq - 1];
+  const int lo = max(0, p_first - window + 1);
+  const int nitems = nq * nh;
+  float* myq = qbuf + wave * D;
+  float* myp = pbuf + wave * 64;
+
+  float m[ATT_ITEMS], l[ATT_ITEMS], acc[ATT_ITEMS][ATT_RPL];
+#pragma unroll
+  for (int i = 0; i < ATT_ITEMS; ++i) {
+    m[i] = -INFINITY;
+    l[i] = 0.f;
+#pragma unroll
+    for (int c = 0; c < ATT_RPL; ++c) acc[i][c] = 0.f;
+  }
+
+  for (int k0 = (lo / KT) * KT; k0 <= p_last; k0 += KT) {
+    __syncthreads();                       // previous tile fully consumed
+    const int rows = min(KT, p_last + 1 - k0);   // only these rows of the tile are staged (and read)
+    {
+      const long base = ((long)bt[(long)s * btw + k0 / PAGE] * PAGE + (k0 % PAGE)) * D;
+      for (int e = threadIdx.x; e < rows * D; e += blockDim.x) {
+        const int j = e / D, d = e - j * D;
+        ktile[j * ldk + d] = cache[base + e];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ii = 0; ii < ATT_ITEMS; ++ii) {
+      const int item = wave + ii * ATT_WAVES;
+      if (item >= nitems) continue;                       // wave-uniform
+      const int tq = item / nh, hh = item - tq * nh;
+      const long row = r0 + t0 + tq;
+      const int h = h0 + hh;
+      const int p = pos[row];
+      const int j = k0 + lane;
+      const bool vis = lane < rows && j <= p && j > p - window;
+      if (__ballot(vis) == 0ull) continue;                // no visible key of this tile
+      // this item's query into the wave's LDS copy
+      {
+        const T* ql = q_lat + (row * H + h) * R;
+        const T* qr = q_rot + (row * H + h) * Dr;
+        for (int d = lane; d < D; d += 64) myq[d] = d < R ? ldf(ql + d) : ldf(qr + d - R);
+      }
+      float sc = -INFINITY;
+      if (vis) {
+        const T* kr = ktile + lane * ldk;
+        float a = 0.f;
+        for (int d = 0; d < D; ++d) a += myq[d] * ldf(kr + d);
+        sc = a * scale;
+      }
+      const float mt = mx_wave_max(sc);
+      const float mn = fmaxf(m[ii], mt);
+      const float corr = expf(m[ii] - mn);                 // exp(-inf) = 0 on the first tile
+      const float pj = vis ? expf(sc - mn) : 0.f;
+      l[ii] = l[ii] * corr + mx_wave_sum(pj);
+      m[ii] = mn;
+      myp[lane] = pj;
+      // one wave writes and reads myq / myp: its LDS accesses complete in program order
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int c = 0; c < ATT_RPL; ++c) {
+        const int d = lane + 64 * c;
+        if (d < R) {
+          float a = acc[ii][c] * corr;
+          for (int jj = 0; jj < rows; ++jj) a += myp[jj] * ldf(ktile + jj * ldk + d);
+          acc[ii][c] = a;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+#pragma unroll
+  for (int ii = 0; ii < ATT_ITEMS; ++ii) {
+    const int item = wave + ii * ATT_WAVES;
+    if (item >= nitems) continue;
+    const int tq = item / nh, hh = item - tq * nh;
+    const long row = r0 + t0 + tq;
+    const int h = h0 + hh;
+    float g = 1.0f / l[ii];
+    if (gate != nullptr) g *= mx_sigmoid(ldf(gate + row * sgate + h));
+#pragma unroll
+    for (int c = 0; c < ATT_RPL; ++c) {
+      const int d = lane + 64 * c;
+      if (d < R) stf(out + (row * H + h) * R + d, acc[ii][c] * g);
+    }
+  }
+}
+
+}  // namespace
+
+// kv [T, R+Dr] slice (row stride skv); q [T, ...] with head h's rotated part at h*q_head_stride+q_rot_off
+// (row stride sq); q_rot out [T, H, Dr]; cache [pages*64, R+Dr]; all of storage type dt
+MX_API int mx_latent_prep(const void* kv, long skv, const float* norm_w, float eps, const float* inv_freq,
+                          int rot_dims, const int* pos, const int* slots, void* cache, const void* q, long sq,
+                          int q_head_stride, int q_rot_off, void* q_rot, int dt, int T, int H, int R, int Dr,
+                          hipStream_t st) {
+  if (T <= 0) return 0;
+  MX_DISPATCH(dt, TT, latent_prep_kernel<TT><<<T, 256, 0, st>>>((const TT*)kv, skv, norm_w, eps, inv_freq, rot_dims,
+                                                                pos, slots, (TT*)cache, (const TT*)q, sq,
+                                                                q_head_stride, q_rot_off, (TT*)q_rot, H, R, Dr));
+  MX_RETURN_LAUNCH();
+}
+
+// q_lat [T, H, R], q_rot [T, H, Dr], out [T, H, R] contiguous; cu [S+1] row bounds of the segments,
+// pos [T] positions, bt [S, btw] page tables; gate [T, >=H] slice (row stride sgate) or null.
+MX_API int mx_latent_attend(const void* q_lat, const void* q_rot, const void* cache, const int* cu, const int* pos,
+                            const int* bt, int btw, const void* gate, long sgate, int window, float scale,
+                            void* out, int dt, int S, int max_len, int H, int R, int Dr, hipStream_t st) {
+  if (S <= 0 || max_len <= 0) return 0;
+  if (R > 64 * ATT_RPL) return (int)hipErrorInvalidValue;
+  const int D = R + Dr;
+  const int esz = dt == 1 ? 4 : 2;
+  // key row stride: odd in 4-byte words
+  int ldk = D;
+  if (esz == 4) ldk += (ldk & 1) ? 0 : 1;
+  else {
+    ldk += ldk & 1;
+    if (((ldk / 2) & 1) == 0) ldk += 2;
+  }
+  int KT = 64;
+  while (KT > 8 && (size_t)KT * ldk * esz > 40 * 1024) KT >>= 1;
+  // decode-like steps (one row per segment): all items are heads; prompt chunks: 4 rows x 8 heads
+  const int QT = max_len == 1 ? 1 : 4;
+  int HB = (ATT_WAVES * ATT_ITEMS) / QT;
+  if (HB > H) HB = H;
+  const size_t lds = (((size_t)KT * ldk * esz + 15) & ~(size_t)15) + (size_t)ATT_WAVES * (D + 64) * sizeof(float);
+  if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
+  dim3 grid((max_len + QT - 1) / QT, (H + HB - 1) / HB, S);
+  MX_DISPATCH(dt, TT, latent_attend_kernel<TT><<<grid, ATT_WAVES * 64, lds, st>>>(
+      (const TT*)q_lat, (const TT*)q_rot, (const TT*)cache, cu, pos, bt, btw, (const TT*)gate, sgate, window, scale,
+      (TT*)out, H, R, Dr, QT, HB, KT, ldk));
+  MX_RETURN_LAUNCH();
+}

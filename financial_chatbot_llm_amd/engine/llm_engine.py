@@ -27,6 +27,7 @@ from .block_manager import make_block_manager
 from .model_runner import CollectiveTimeout, ModelRunner, StepInputs, build_step_inputs, sample_rows
 from .scheduler import Scheduler, StepCostModel
 from .sequence import PENDING, SamplingParams, Sequence, SeqStatus
+from .state_manager import StateSlotPool
 from .speculative import PromptLookup, accept_draft
 from .tokenizer import BaseTokenizer, load_tokenizer
 
@@ -46,7 +47,10 @@ class StepOutput:
 def plan_kv_blocks(cfg: EngineConfig, model, device) -> int:
     if cfg.num_kv_blocks:
         return cfg.num_kv_blocks
-    per_block = KVCache.bytes_per_block(model.cfg.num_layers, model.hkv, model.D)
+    if hasattr(model, "kv_bytes_per_block"):
+        per_block = model.kv_bytes_per_block()
+    else:
+        per_block = KVCache.bytes_per_block(model.cfg.num_layers, model.hkv, model.D)
     if device.type != "cuda":
         return max(64, (cfg.max_num_seqs * cfg.max_model_len // KV_BS) // 8)
     free, _ = torch.cuda.mem_get_info(device)
@@ -70,9 +74,16 @@ class LLMEngine:
         self.tokenizer = tokenizer or load_tokenizer(cfg.tokenizer, self.model.cfg.vocab_size)
         self.eos_ids = set(self.tokenizer.eos_ids)
         nblocks = plan_kv_blocks(cfg, self.model, device)
-        self.kv = KVCache(self.model.cfg.num_layers, nblocks, self.model.hkv, self.model.D,
-                          dtype=getattr(self.model, "dtype", torch.bfloat16), device=device)
-        self.bm = make_block_manager(nblocks, KV_BS, cfg.enable_prefix_caching)
+        # recurrent layers: one state slot per running sequence; their state cannot be rebuilt from a
+        # cached prefix or rolled back over rejected draft rows, so both are off for such models
+        self.stateful = bool(getattr(self.model, "has_state", False))
+        self.state_slots = StateSlotPool(cfg.max_num_seqs) if self.stateful else None
+        if hasattr(self.model, "make_cache"):
+            self.kv = self.model.make_cache(nblocks, cfg.max_num_seqs)
+        else:
+            self.kv = KVCache(self.model.cfg.num_layers, nblocks, self.model.hkv, self.model.D,
+                              dtype=getattr(self.model, "dtype", torch.bfloat16), device=device)
+        self.bm = make_block_manager(nblocks, KV_BS, cfg.enable_prefix_caching and not self.stateful)
         base, per_row, per_tok = cfg.step_cost_ms
         self.scheduler = Scheduler(self.bm, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.max_model_len,
                                    token_quantum=cfg.step_token_quantum if device.type == "cuda" else 0,
@@ -83,7 +94,8 @@ class LLMEngine:
                                    sjf_tokens=getattr(cfg, "sched_sjf_tokens", 0),
                                    sjf_step_cap=getattr(cfg, "sched_sjf_step_cap", 0),
                                    short_reserve_tokens=getattr(cfg, "sched_short_reserve_tokens", 0),
-                                   short_first=getattr(cfg, "sched_short_first", False))
+                                   short_first=getattr(cfg, "sched_short_first", False),
+                                   state_slots=self.state_slots)
         self.runner = ModelRunner(self.model, self.kv, cfg.max_model_len, max_decode_batch=cfg.max_num_seqs,
                                   use_graphs=cfg.use_cuda_graph, graph_sizes=cfg.graph_batch_sizes)
         self.requests: Dict[str, Sequence] = {}
@@ -271,7 +283,7 @@ class LLMEngine:
         max_model_len or the teacher-forced output's last token; cut before any stop token (the
         model's own stop token then arrives as the bonus sample and ends the sequence as usual)."""
         p = seq.params
-        if p.prompt_lookup <= 0 or seq.finished:
+        if p.prompt_lookup <= 0 or seq.finished or self.stateful:
             return []
         k = len(seq.output_ids) + len(after)
         room = min(p.prompt_lookup, MAX_DRAFT, p.max_tokens - k - 1, self.cfg.max_model_len - seq.num_tokens - len(after) - 2)
@@ -621,6 +633,55 @@ class LLMEngine:
             raise RuntimeError("cp_follower_loop needs cp_size > 1 and init_cp_groups")
         self.cp.follower_loop()
 
+    # -- trace replay -------------------------------------------------------------------
+    def replay_step(self, entries, end: Seq[str] = ()) -> torch.Tensor:
+        """Run one externally dictated step and return logits instead of sampling.
+
+        ``entries``: (request id, next token ids, wanted places among them) per request, all one
+        batch; a request is admitted at its first entry and may sit out steps.  ``end``: requests
+        finished after this step (pages and state slot go back to the pools).  Returns f32 logits
+        [wanted places, vocab] on the CPU, in the order of the entries and their places.  The step
+        goes through the scheduler's admission (:meth:`Scheduler.schedule_replay`), the block and
+        state-slot managers, ``build_step_inputs`` and the runner's forward like a scheduled one."""
+        import numpy as np
+        if self._inflight is not None:
+            raise RuntimeError("replay_step cannot interleave with step()")
+        plan = []
+        for rid, toks, _ in entries:
+            seq = self.requests.get(rid)
+            if seq is None:
+                seq = Sequence(rid, [], SamplingParams(temperature=0.0, max_tokens=1 << 30, ignore_eos=True))
+                self.requests[rid] = seq
+            if seq.num_tokens + len(toks) > self.cfg.max_model_len:
+                raise ValueError(f"{rid}: longer than max_model_len {self.cfg.max_model_len}")
+            seq.prompt_ids.extend(int(t) for t in toks)
+            plan.append((seq, len(toks)))
+        batch = self.scheduler.schedule_replay(plan)
+        si = build_step_inputs(batch)
+        first_row, off = {}, 0
+        for seq, _, n in batch.prefill:
+            first_row[id(seq)] = off
+            off += n
+        for j, seq in enumerate(batch.decode):
+            first_row[id(seq)] = off + j
+        rows = [first_row[id(seq)] + int(w) for (seq, n), (_, _, want) in zip(plan, entries) for w in want]
+        for (seq, n), (_, _, want) in zip(plan, entries):
+            if any(not 0 <= int(w) < n for w in want):
+                raise ValueError(f"{seq.request_id}: a wanted place is outside the step's tokens")
+        si.logits_idx = np.asarray(rows, np.int64)
+        logits = self.runner.logits_at(si)
+        for seq, start, n in batch.prefill:
+            seq.num_computed = start + n
+            self.bm.commit(seq)
+        for seq in batch.decode:
+            seq.num_computed = seq.num_tokens
+            self.bm.commit(seq)
+        for rid in end:
+            seq = self.requests.pop(rid, None)
+            if seq is not None:
+                self.scheduler.finish(seq, "stop")
+        return logits
+
     # -- convenience --------------------------------------------------------------------
     def generate(self, prompts: Seq[Seq[int]], params: SamplingParams) -> List[List[int]]:
         seqs = [self.add_request(f"gen-{i}-{id(p)}", p, params) for i, p in enumerate(prompts)]
@@ -671,5 +732,6 @@ class LLMEngine:
         g = float(1 << 30)
         return {"hbm_used_gib": round((total - free) / g, 1), "hbm_total_gib": round(total / g, 1),
                 "torch_peak_reserved_gib": round(torch.cuda.max_memory_reserved(self.device) / g, 1),
-                "kv_pool_gib": round(self.bm.num_blocks * KVCache.bytes_per_block(
-                    self.model.cfg.num_layers, self.model.hkv, self.model.D) / g, 1)}
+                "kv_pool_gib": round(self.bm.num_blocks * (
+                    self.model.kv_bytes_per_block() if hasattr(self.model, "kv_bytes_per_block") else
+                    KVCache.bytes_per_block(self.model.cfg.num_layers, self.model.hkv, self.model.D)) / g, 1)}

@@ -57,6 +57,7 @@ class StepInputs:
     top_p: np.ndarray               # [S]
     src: Optional[np.ndarray] = None  # [Bd] row of the previous step's sampled vector (-1: ids[] is real)
     pwork: Optional[np.ndarray] = None  # prefill attention work list (filled by the runner): [n, 2] or lean [., 6]
+    sslots: Optional[np.ndarray] = None  # [Sp + Bd] recurrent-state slot per sequence of the step (stateful models)
 
     @property
     def num_prefill_tokens(self) -> int:
@@ -64,7 +65,7 @@ class StepInputs:
 
     # -- C4 wire format: one flat byte buffer (no pickling) ------------------------------------
     _ARRAYS = ("ids", "positions", "slots", "cu_q", "ctx_p", "bt_p", "ctx_d", "bt_d", "logits_idx", "temps",
-               "seeds", "top_k", "top_p", "src", "pwork")
+               "seeds", "top_k", "top_p", "src", "pwork", "sslots")
 
     def pack(self) -> np.ndarray:
         """[header int64: max_q_len, then (dtype code, rows, cols) per array] + raw array bytes."""
@@ -202,6 +203,8 @@ def build_step_inputs(batch: ScheduledBatch) -> StepInputs:
     i32 = lambda x: np.asarray(x, np.int32)  # noqa: E731
     cat = lambda parts, tail: np.concatenate(parts + [i32(tail)]) if parts else i32(tail)  # noqa: E731
     src_a = i32(src) if any(x >= 0 for x in src) else None
+    seqs = [q for q, _, _ in batch.prefill] + list(batch.decode)
+    sslots = i32([q.state_slot for q in seqs]) if any(q.state_slot >= 0 for q in seqs) else None
     bt_d = _table(tables_d)
     if _attn.LEAN_FLAGS & 1 and _attn.DECODE_LEAN and len(ctx_d) >= _attn.LEAN_NT_MIN_B:
         # the lean kernel's cache policy per block -- only where ops.decode keeps the NT bit
@@ -209,7 +212,7 @@ def build_step_inputs(batch: ScheduledBatch) -> StepInputs:
     return StepInputs(cat(ids_parts, ids_d), cat(pos_parts, pos_d), cat(slot_parts, slots_d), i32(cu), i32(ctx_p),
                       _table(tables_p), max_q, i32(ctx_d), bt_d, np.asarray(logits_idx, np.int64),
                       np.asarray(temps, np.float32), np.asarray(seeds, np.int64), i32(tk), np.asarray(tp, np.float32),
-                      src_a)
+                      src_a, sslots=sslots)
 
 
 class CollectiveTimeout(RuntimeError):
@@ -266,11 +269,14 @@ class ModelRunner:
         self.on_gpu = self.device.type == "cuda"
         self.use_graphs = use_graphs and self.on_gpu
         self.G = model.hq // model.hkv
+        # layered decoders (models.gezavik) take the step as segments (AttentionMetadata.seg_*) and bring
+        # their own attention kernels: no decode workspace, no prefill work lists
+        self.seg = bool(getattr(model, "segment_meta", False))
         self.graph_sizes = tuple(sorted(s for s in graph_sizes if s <= max_decode_batch))
         self.max_decode_batch = max(self.graph_sizes) if self.graph_sizes else max_decode_batch
         cfg = model.cfg
         self.decode_ws = DecodeWorkspace.create(max(max_decode_batch, 1), model.hq, model.D, max_model_len,
-                                                self.device) if self.on_gpu else None
+                                                self.device) if self.on_gpu and not self.seg else None
         # TP decode as two micro-batch chains on two streams (DecoderModel.forward_decode_dual): their
         # all-reduces hide under the other chain's compute; needs the second custom-AR channel
         # (decided at the first graph capture: the engine enables the AR channels after building us)
@@ -365,12 +371,14 @@ class ModelRunner:
     def _meta(self, si: StepInputs, slots: torch.Tensor) -> AttentionMetadata:
         m = AttentionMetadata(slots=slots, num_prefill_tokens=si.num_prefill_tokens, num_decode=si.num_decode,
                               decode_ws=self.decode_ws)
+        if self.seg:
+            self._segments(si, m)
         if si.num_prefill_tokens:
             m.cu_q = self._to_dev(si.cu_q)
             m.ctx_lens_p = self._to_dev(si.ctx_p)
             m.block_tables_p = self._to_dev(si.bt_p)
             m.max_q_len = si.max_q_len
-            if self.on_gpu:   # LPT-ordered prefill attention tiles (staged with the step when precomputed)
+            if self.on_gpu and not self.seg:   # LPT-ordered prefill attention tiles (staged with the step when precomputed)
                 work = si.pwork if si.pwork is not None else prefill_plan(si.cu_q, si.ctx_p, self.G, self.model.hkv)
                 m.prefill_work = self._to_dev(work) if work is not None else None
                 if work is not None and work.shape[1] == 6:        # lean split-KV list: its counts
@@ -379,6 +387,23 @@ class ModelRunner:
             m.ctx_lens_d = self._to_dev(si.ctx_d)
             m.block_tables_d = self._to_dev(si.bt_d)
         return m
+
+    def _segments(self, si: StepInputs, m: AttentionMetadata) -> None:
+        """The step as segments: each prefill chunk, then each decode row, with one page table and
+        one state slot per segment."""
+        sp, bd = len(si.ctx_p), si.num_decode
+        tp = si.num_prefill_tokens
+        cu = np.concatenate([si.cu_q[:sp + 1] if sp else np.zeros(1, np.int32),
+                             tp + 1 + np.arange(bd, dtype=np.int32)]).astype(np.int32)
+        w = max(si.bt_p.shape[1] if sp else 1, si.bt_d.shape[1] if bd else 1)
+        bt = np.zeros((sp + bd, w), np.int32)
+        if sp:
+            bt[:sp, :si.bt_p.shape[1]] = si.bt_p
+        if bd:
+            bt[sp:, :si.bt_d.shape[1]] = np.where(si.bt_d < 0, -si.bt_d - 1, si.bt_d)   # undo shared-block marks
+        ss = si.sslots if si.sslots is not None else np.full(sp + bd, -1, np.int32)
+        m.seg_cu, m.seg_bt, m.seg_state = self._to_dev(cu), self._to_dev(bt), self._to_dev(ss)
+        m.seg_max_len = max(si.max_q_len if sp else 0, 1 if bd else 0)
 
     def _gather_pending(self, ids: torch.Tensor, src: torch.Tensor, offset: int) -> None:
         """ids[offset + r] <- last_sampled[src[r]] where src[r] >= 0 (device-side, no host sync)."""
@@ -437,11 +462,28 @@ class ModelRunner:
         idx = self._to_dev(si.logits_idx)
         return self.model.logits(h.index_select(0, idx))
 
+    def logits_at(self, si: StepInputs) -> torch.Tensor:
+        """Run the step and return the f32 logits of its ``logits_idx`` rows on the CPU ([0, V] when
+        no row is asked for: the step still runs and leaves its cache and state)."""
+        self.stats["steps"] += 1
+        self.stats["tokens"] += len(si.ids)
+        self._stage_inputs(si)
+        try:
+            if len(si.logits_idx) == 0:
+                self._forward_only(si)
+                out = torch.zeros((0, self.model.cfg.vocab_size), dtype=torch.float32)
+            else:
+                out = self.forward_logits(si).float().cpu()
+        finally:
+            self._staged = None
+        return out
+
     def _fused_sampling(self, h: torch.Tensor) -> bool:
         """Does sampling the rows ``h`` run inside the LM head (fused K11 + K12)?  TP=1 only: under TP
         the vocabulary is sharded and the logits are all-gathered before sampling."""
         m = self.model
-        return getattr(m, "tp_size", 1) == 1 and hasattr(m, "lm_weight") and ops.fused_lm_head_ok(h, m.lm_weight())
+        return (getattr(m, "tp_size", 1) == 1 and hasattr(m, "lm_weight") and h.dtype == torch.bfloat16
+                and ops.fused_lm_head_ok(h, m.lm_weight()))
 
     def _lm_tiled(self):
         f = getattr(self.model, "lm_tiled", None)
@@ -528,7 +570,7 @@ class ModelRunner:
             graph = True
         else:
             with marker(f"forward.eager[{len(si.ids)}]"):
-                if si.num_prefill_tokens and si.pwork is None and self.on_gpu:
+                if si.num_prefill_tokens and si.pwork is None and self.on_gpu and not self.seg:
                     si.pwork = prefill_plan(si.cu_q, si.ctx_p, self.G, self.model.hkv)
                 self._stage_inputs(si)
                 try:
@@ -578,25 +620,29 @@ class ModelRunner:
         # by ONE pinned H2D copy
         self._src_off = 4 * B + B * W          # pending-token gather rows (-1: host id)
         self._topk_off = self._src_off + B     # per-row top-k (0: off)
-        self._dev_i32 = torch.zeros(self._topk_off + B, dtype=torch.int32, device=self.device)
+        self._sslot_off = self._topk_off + B   # per-row recurrent-state slot (-1: padding row)
+        self._dev_i32 = torch.zeros(self._sslot_off + B, dtype=torch.int32, device=self.device)
         d = self._dev_i32
         self._static = {
             "ids": d[0:B], "pos": d[B:2 * B], "slots": d[2 * B:3 * B], "ctx": d[3 * B:4 * B],
             "bt": d[4 * B:self._src_off].view(B, W),
             "src": d[self._src_off:self._topk_off],
             "top_k": d[self._topk_off:self._topk_off + B],
+            "sslot": d[self._sslot_off:self._sslot_off + B],
+            "seg_cu": torch.arange(B + 1, dtype=torch.int32, device=self.device),
             "f32": torch.zeros(2 * B, dtype=torch.float32, device=self.device),     # temps | top_p
             "seeds": torch.zeros(B, dtype=torch.int64, device=self.device),
         }
         self._static["slots"].fill_(-1)
         self._static["ctx"].fill_(1)
         self._static["src"].fill_(-1)
+        self._static["sslot"].fill_(-1)
         self._static["temps"], self._static["top_p"] = self._static["f32"][:B], self._static["f32"][B:]
         self._static["top_p"].fill_(1.0)
         # two pinned staging sets, alternated per graph step: in overlap mode the host packs step
         # N+1 while step N's H2D copy may still be queued behind step N-1 on the stream, so a
         # single buffer could be overwritten before the DMA reads it
-        self._pinned_sets = [(torch.zeros(self._topk_off + B, dtype=torch.int32).pin_memory(),
+        self._pinned_sets = [(torch.zeros(self._sslot_off + B, dtype=torch.int32).pin_memory(),
                               torch.zeros(2 * B, dtype=torch.float32).pin_memory(),
                               torch.zeros(B, dtype=torch.int64).pin_memory()) for _ in range(2)]
         self._pin_flip = 0
@@ -637,6 +683,9 @@ class ModelRunner:
         else:
             meta = AttentionMetadata(slots=s["slots"][:B], num_prefill_tokens=0, num_decode=B,
                                      ctx_lens_d=s["ctx"][:B], block_tables_d=s["bt"][:B], decode_ws=self.decode_ws)
+            if self.seg:     # one segment per row; padding rows carry slot -1, position 0, page 0
+                meta.seg_cu, meta.seg_bt, meta.seg_state = s["seg_cu"][:B + 1], s["bt"][:B], s["sslot"][:B]
+                meta.seg_max_len = 1
             h = self.model.forward(s["ids"][:B], s["pos"][:B], meta, self.kv)
         if not filtered:
             if self._shard_sampling():     # TP: top-k / top-p rows of this bucket replay eagerly
@@ -739,7 +788,12 @@ class ModelRunner:
         buf = self._pinned_i32.numpy()
         # layout: ids | pos | slots | ctx | bt  (each section sized for the largest bucket)
         buf[0:n] = si.ids
+        buf[S:S + B] = 0
         buf[S:S + n] = si.positions
+        ss = buf[self._sslot_off:self._sslot_off + S]
+        ss[:B] = -1
+        if si.sslots is not None:
+            ss[:n] = si.sslots
         buf[2 * S:2 * S + B] = -1
         buf[2 * S:2 * S + n] = si.slots
         buf[3 * S:3 * S + B] = 1

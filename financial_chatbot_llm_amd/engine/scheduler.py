@@ -85,8 +85,11 @@ class Scheduler:
                  aging_s: float = 1.0, clock=time.perf_counter, token_quantum: int = 0,
                  cost_model: "StepCostModel" = None, burst_tokens: int = 0, burst_age_s: float = 0.5,
                  sjf_tokens: int = 0, sjf_step_cap: int = 0, short_reserve_tokens: int = 0,
-                 short_first: bool = False):
+                 short_first: bool = False, state_slots=None):
         self.bm = block_manager
+        # models with recurrent layers: a sequence holds one state slot (engine.state_manager) from
+        # admission until it finishes, is aborted or is preempted
+        self.slots = state_slots
         self.max_num_seqs = max_num_seqs
         self.max_num_batched_tokens = max_num_batched_tokens
         self.max_model_len = max_model_len
@@ -152,6 +155,10 @@ class Scheduler:
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
 
+    def _release_state(self, seq: Sequence) -> None:
+        if self.slots is not None:
+            self.slots.release(seq)
+
     def abort(self, seq: Sequence) -> None:
         if seq in self.running:
             self.running.remove(seq)
@@ -160,6 +167,7 @@ class Scheduler:
             self.waiting.remove(seq)
             if seq.block_table:
                 self.bm.free(seq)
+        self._release_state(seq)
         seq.status = SeqStatus.FINISHED
 
     def _preempt(self, seq: Sequence, batch: ScheduledBatch) -> None:
@@ -167,6 +175,7 @@ class Scheduler:
             seq.drop_draft()                # not launched: recomputed later without it
         self.running.remove(seq)
         self.bm.free(seq)
+        self._release_state(seq)          # recomputed from position 0: any slot will do then
         seq.num_computed = 0
         seq.status = SeqStatus.WAITING
         seq.num_preemptions += 1
@@ -279,11 +288,16 @@ class Scheduler:
             if not seq.block_table:
                 self.bm.match_prefix(seq)
             n = min(seq.remaining_prefill, budget)
+            if self.slots is not None and seq.state_slot < 0 and self.slots.num_free() == 0:
+                stop = "seqs"          # every state slot is held by a running sequence
+                break
             if not self.bm.grow(seq, seq.num_computed + n):
                 if seq.block_table and not self.running:
                     raise MemoryError("KV pool too small for a single prompt")
                 stop = "grow"
                 break
+            if self.slots is not None:
+                self.slots.acquire(seq)
             self.waiting.popleft()
             tok_admit[seq.params.max_tokens > self.short_output_tokens] += n
             if seq.admit_time is None:
@@ -321,8 +335,12 @@ class Scheduler:
             n = seq.remaining_prefill
             if n > self.sjf_tokens or n > budget or n > cap:
                 continue
+            if self.slots is not None and seq.state_slot < 0 and self.slots.num_free() == 0:
+                break
             if not self.bm.grow(seq, seq.num_computed + n):
                 break
+            if self.slots is not None:
+                self.slots.acquire(seq)
             self.waiting.remove(seq)
             if seq.admit_time is None:
                 seq.admit_time = now
@@ -385,3 +403,32 @@ class Scheduler:
         elif seq in self.waiting:          # preempted while its last token was in flight
             self.waiting.remove(seq)
         self.bm.free(seq, evict_first=seq.params.ephemeral_kv)
+        self._release_state(seq)
+
+    def schedule_replay(self, plan: List[Tuple[Sequence, int]]) -> ScheduledBatch:
+        """One step whose rows are dictated from outside (trace replay): ``plan`` lists, in batch
+        order, each sequence and how many of its not yet computed tokens run now.  Admission, page
+        growth and state slots go through the same managers as :meth:`schedule`; a single next token
+        of a sequence that has computed tokens is a decode row, everything else a prefill chunk.
+        Nothing is preempted: a plan that does not fit raises."""
+        batch = ScheduledBatch()
+        for seq, n in plan:
+            if n <= 0 or n > seq.remaining_prefill:
+                raise ValueError(f"{seq.request_id}: {n} tokens asked, {seq.remaining_prefill} pending")
+            if seq.status == SeqStatus.WAITING:
+                if len(self.running) >= self.max_num_seqs:
+                    raise MemoryError("more live sequences than max_num_seqs")
+                if self.slots is not None and not self.slots.acquire(seq):
+                    raise MemoryError("no free state slot")
+                if seq in self.waiting:
+                    self.waiting.remove(seq)
+                seq.status = SeqStatus.RUNNING
+                self.running.append(seq)
+            if not self.bm.grow(seq, seq.num_computed + n):
+                raise MemoryError("KV pool too small for the replayed step")
+            if n == 1 and seq.num_computed > 0 and seq.remaining_prefill == 1:
+                batch.decode.append(seq)
+            else:
+                batch.prefill.append((seq, seq.num_computed, n))
+        # the flat batch is prefill rows first, then decode rows
+        return batch

@@ -61,6 +61,7 @@ class Sequence:
         self.params = params
         self.status = SeqStatus.WAITING
         self.block_table: List[int] = []
+        self.state_slot = -1           # recurrent-state slot (engine.state_manager; -1: none)
         self.num_computed = 0          # tokens whose KV is in the cache
         self.num_cached_prompt = 0     # prefix-cache hit (tokens)
         self.num_prefilled = 0         # tokens run through prefill chunks (recomputes included)

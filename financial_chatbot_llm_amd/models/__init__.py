@@ -10,6 +10,8 @@ def build_model(engine_cfg, device, seed: int = 0):
     from .llama import LlamaModel
     from .mixtral import MixtralModel
     cfg = get_model_config(engine_cfg.model)
+    if cfg.arch == "gezavik":
+        return _build_layered(cfg, engine_cfg, device, seed)
     if cfg.arch == "mixtral":
         model = MixtralModel(cfg, device=device, fp8=getattr(engine_cfg, "dtype", "bf16") == "fp8",
                              moe_parallel=getattr(engine_cfg, "moe_parallel", "tp"))
@@ -26,6 +28,33 @@ def build_model(engine_cfg, device, seed: int = 0):
         load_decoder_weights(model, engine_cfg.weights)
         if cfg.arch == "mixtral" and model.fp8:
             model.quantize_experts()          # checkpoint experts (bf16) -> tiled fp8 + row scales
+    else:
+        model.init_random(seed=engine_cfg.seed if hasattr(engine_cfg, "seed") else seed)
+    return model
+
+
+def _build_layered(cfg, engine_cfg, device, seed: int):
+    """Layered decoders run in bf16 (f32 statistics, state and residual stream) or, with
+    ``dtype="fp32"``, in true f32 throughout; their checkpoint is the model directory itself."""
+    import os
+
+    import torch
+
+    from .gezavik import GezavikModel
+    from .weights import read_safetensors
+    if getattr(engine_cfg, "tp_size", 1) > 1:
+        raise ValueError(f"{cfg.name}: tensor parallelism is not implemented for layered decoders")
+    dtype = str(getattr(engine_cfg, "dtype", "bf16")).lower()
+    if dtype not in ("bf16", "bfloat16", "fp32", "float32"):
+        raise ValueError(f"{cfg.name}: dtype must be bf16 or fp32, got {dtype!r}")
+    f32 = dtype in ("fp32", "float32")
+    if f32:      # no reduced-precision matrix mode for f32 products
+        torch.backends.cuda.matmul.allow_tf32 = False
+        torch.backends.cudnn.allow_tf32 = False
+    model = GezavikModel(cfg, device=device, dtype=torch.float32 if f32 else torch.bfloat16)
+    src = engine_cfg.weights or (engine_cfg.model if os.path.isdir(engine_cfg.model) else None)
+    if src:
+        model.load_state(read_safetensors(src))
     else:
         model.init_random(seed=engine_cfg.seed if hasattr(engine_cfg, "seed") else seed)
     return model

@@ -15,7 +15,7 @@ from typing import Dict, Optional
 @dataclass(frozen=True)
 class ModelConfig:
     name: str
-    arch: str                       # "llama" | "mixtral" | "bert"
+    arch: str                       # "llama" | "mixtral" | "bert" | "gezavik"
     vocab_size: int
     hidden_size: int
     num_layers: int
@@ -34,6 +34,10 @@ class ModelConfig:
     bos_token_id: int = 128000
     eos_token_ids: tuple = (128001, 128009)
     pad_token_id: int = 0
+    # layered (hybrid) decoders: one entry per layer, {"type": mixer kind, "mixer": {...}, "mlp": {...} | None},
+    # as the checkpoint's config.json gives them; residual_mult scales each block's update
+    layers: tuple = ()
+    residual_mult: float = 1.0
 
     @property
     def q_size(self) -> int:
@@ -73,7 +77,16 @@ REGISTRY: Dict[str, ModelConfig] = {
 }
 
 
+def _register_layered() -> None:
+    from .gezavik import example_config
+    for name, kw in (("gezavik-tiny", dict(width=192, vocab=1024, heads=3, pattern="amAm")),
+                     ("gezavik-1b", dict(width=2048, vocab=32768, heads=16, pattern="aMmAmMaM" * 2, scale_up=True))):
+        REGISTRY[name] = layered_config(example_config(**kw), name)
+
+
 def get_model_config(name: str) -> ModelConfig:
+    if name.startswith("gezavik-") and name not in REGISTRY:
+        _register_layered()
     if name in REGISTRY:
         return REGISTRY[name]
     if os.path.isdir(name) and os.path.exists(os.path.join(name, "config.json")):
@@ -84,6 +97,8 @@ def get_model_config(name: str) -> ModelConfig:
 def from_hf(path: str, name: Optional[str] = None) -> ModelConfig:
     with open(path) as fh:
         c = json.load(fh)
+    if "architecture" in c:          # layered decoders name their design and list their layers
+        return layered_config(c, name)
     mt = c.get("model_type", "llama")
     if mt == "bert":
         return ModelConfig(name or "hf-bert", "bert", c["vocab_size"], c["hidden_size"], c["num_hidden_layers"],
@@ -103,3 +118,23 @@ def from_hf(path: str, name: Optional[str] = None) -> ModelConfig:
         rope_scaling=c.get("rope_scaling"), norm_eps=c.get("rms_norm_eps", 1e-5),
         tie_embeddings=c.get("tie_word_embeddings", False), num_experts=c.get("num_local_experts", 0),
         top_k_experts=c.get("num_experts_per_tok", 0), bos_token_id=c.get("bos_token_id", 1), eos_token_ids=eos)
+
+
+LAYERED_ARCHS = ("gezavik",)
+
+
+def layered_config(c: Dict, name: Optional[str] = None) -> ModelConfig:
+    """A layered decoder's ``config.json`` (``architecture``, ``layers``: type / mixer / mlp per layer,
+    ``norm.eps``, ``residual_mult``, ``vocab``, ``width``) -> :class:`ModelConfig`.  The flat head
+    fields hold the first attention layer's sizes (informational; the layers carry their own)."""
+    arch = str(c["architecture"]).lower()
+    if arch not in LAYERED_ARCHS:
+        raise ValueError(f"unknown layered architecture {c['architecture']!r}; known: {LAYERED_ARCHS}")
+    layers = tuple(c["layers"])
+    att = next((l["mixer"] for l in layers if "heads" in l["mixer"] and "kv_rank" in l["mixer"]), None)
+    heads = att["heads"] if att else 1
+    hd = (att["dim"] + att["rot_dim"]) if att else c["width"]
+    ffs = [l["mlp"]["ff"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "dense"]
+    return ModelConfig(name or arch, arch, c["vocab"], c["width"], len(layers), heads, 1, hd, max(ffs, default=0),
+                       max_position=1 << 24, norm_eps=float(c["norm"]["eps"]), bos_token_id=0, eos_token_ids=(),
+                       layers=layers, residual_mult=float(c.get("residual_mult", 1.0)))

@@ -81,6 +81,56 @@ _SIGS = {
 }
 
 
+c_double = ctypes.c_double
+# libpenny_mixers.so (csrc/mixers): the sequence-mixer kernels of the hybrid decoders, a library of
+# its own -- a model that runs only these builds and loads only these
+_MIXER_SIGS = {
+    "mx_embed": [P, P, c_int, P, c_int, c_int, c_int, P],
+    "mx_residual_norm": [P, P, c_long, P, c_long, c_int, c_float, P, c_float, P, c_int, c_int, c_int, P],
+    "mx_group_norm": [P, c_long, c_int, P, c_long, c_int, P, c_float, P, c_long, c_int, c_int, c_int, c_int, P],
+    "mx_relu2": [P, c_long, P, c_long, c_int, c_int, c_int, P],
+    "mx_glu_clamp": [P, c_long, P, c_long, c_float, c_float, P, c_long, c_int, c_int, c_int, P],
+    "mx_route_biased": [P, P, c_int, c_int, P, P, c_int, P],
+    "mx_moe_combine": [P, P, P, P, P, c_long, P, c_long, c_int, c_int, c_int, P, c_int, c_int, P],
+    "mx_conv_silu": [P, c_long, c_int, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, P],
+    "mx_ssm_scan": [P, c_int, P, c_long, c_int, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mx_latent_prep": [P, c_long, P, c_float, P, c_int, P, P, P, P, c_long, c_int, c_int, P, c_int, c_int, c_int,
+                       c_int, c_int, P],
+    "mx_latent_attend": [P, P, P, P, P, P, c_int, P, c_long, c_int, c_float, P, c_int, c_int, c_int, c_int, c_int,
+                         c_int, P],
+}
+_MIXER_LIB: Optional[ctypes.CDLL] = None
+
+
+def load_mixers(build_if_missing: bool = True) -> ctypes.CDLL:
+    global _MIXER_LIB
+    if _MIXER_LIB is not None:
+        return _MIXER_LIB
+    with _LOCK:
+        if _MIXER_LIB is not None:
+            return _MIXER_LIB
+        from .._build import MIXER_LIB, build_mixers
+        if not os.path.exists(MIXER_LIB) and build_if_missing:
+            build_mixers()
+        try:
+            lib = ctypes.CDLL(MIXER_LIB, mode=ctypes.RTLD_GLOBAL)
+        except OSError as e:
+            raise RuntimeError(f"penny mixer kernel library unavailable: {e}") from e
+        for name, args in _MIXER_SIGS.items():
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = c_int
+        _MIXER_LIB = lib
+        return lib
+
+
+def mcall(name: str, *args) -> None:
+    """Launch a kernel of the mixer library on the current stream."""
+    rc = getattr(load_mixers(), name)(*args)
+    if rc != 0:
+        raise RuntimeError(f"{name} failed with hipError {rc}")
+
+
 def lib_path() -> str:
     """The production kernel library, or its bounds-checked debug build with PENNY_KERNEL_DEBUG=1.
     ``PENNY_KERNEL_LIB`` names another build of the same library (whole-library A/B runs)."""
