@@ -87,6 +87,12 @@ def parse(argv=None):
                          "the step's all-reduce volume priced at stated xGMI rates -- a projection, never a "
                          "multi-GPU measurement")
     ap.add_argument("--json-out", default="")
+    ap.add_argument("--model-throughput", default="", metavar="DESIGN", choices=["", "gezavik"],
+                    help="instead of the serving workload: prefill and decode tokens/s of the named layered design at "
+                         "a few layer sizes beside a Llama twin of equal size (bench/model_throughput.py; one JSON "
+                         "line per model and workload)")
+    from financial_chatbot_llm_amd.bench.model_throughput import add_arguments
+    add_arguments(ap)
     return ap.parse_args(argv)
 
 
@@ -357,6 +363,10 @@ def tp_shard_projection(args, res, tmax: float, turns: int) -> dict:
 
 def main(argv=None) -> int:
     args = parse(argv)
+    if args.model_throughput:
+        os.environ.setdefault("LOG_LEVEL", "WARNING")
+        from financial_chatbot_llm_amd.bench.model_throughput import run as run_model_throughput
+        return run_model_throughput(args)
     launched = "WORLD_SIZE" in os.environ
     if args.gpus < 1:
         log(f"error: --gpus {args.gpus}")

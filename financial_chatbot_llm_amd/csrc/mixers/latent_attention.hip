@@ -12,6 +12,8 @@
 //   mx_latent_attend  windowed causal softmax attention: query at position p sees keys j with
 //                     0 <= p - j < window.  Scores, softmax and accumulation in f32.  The head's
 //                     output is multiplied by sigmoid(gate[t, h]) when a gate is given.
+#include <stdlib.h>
+
 #include "mx_common.h"
 
 namespace {
@@ -194,7 +196,182 @@ latent_attend_kernel(const T* __restrict__ q_lat, const T* __restrict__ q_rot, c
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// bf16 on the matrix cores (v_mfma_f32_16x16x32_bf16).  A block owns 64 (row, head) pairs of one
+// segment -- QT consecutive rows x HB heads, 16 pairs per wave -- and walks the key tiles of the
+// union of their windows, KT = 32 keys at a time.  Per tile and wave:
+//     S^T = K . Q^T      A: key rows from LDS (16-byte reads), B: the wave's queries, in registers
+//     online softmax     the statistics of query (lane % 16) live in that lane, f32
+//     O^T += V^T . P^T   A: the latent part of the tile, transposed in LDS; B: P straight from the
+//                        S^T registers (the MFMA's k slots 8g+i / 8g+4+i hold keys 4g+i / 16+4g+i)
+// Feature dimensions are zero-padded to multiples of 32 (keys) / 16 (values) in LDS and registers.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int MKT = 32;             // keys per tile
+constexpr int MLDV = MKT + 8;       // row stride of the transposed value tile
+
+template <int KSM, int NTM>         // up to 32*KSM key dims, 16*NTM value dims
+__global__ void __launch_bounds__(256)
+latent_attend_mfma_kernel(const bf16* __restrict__ q_lat, const bf16* __restrict__ q_rot,
+                          const bf16* __restrict__ cache, const int* __restrict__ cu, const int* __restrict__ pos,
+                          const int* __restrict__ bt, int btw, const bf16* __restrict__ gate, long sgate, int window,
+                          float scale, bf16* __restrict__ out, int H, int R, int Dr, int QT, int HB) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int D = R + Dr;
+  const int KS = (D + 31) / 32, NT = (R + 15) / 16;
+  const int ldk = KS * 32 + 8;
+  bf16* kt_lds = reinterpret_cast<bf16*>(smem);                 // [MKT][ldk]
+  bf16* vt_lds = kt_lds + MKT * ldk;                            // [NT*16][MLDV]
+  const int s = blockIdx.z;
+  const int r0 = cu[s], n = cu[s + 1] - r0;
+  const int t0 = blockIdx.x * QT;
+  if (t0 >= n) return;
+  const int nq = min(QT, n - t0);
+  const int h0 = blockIdx.y * HB;
+  const int nh = min(HB, H - h0);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
+  const int p_first = pos[r0 + t0], p_last = pos[r0 + t0 + nq - 1];
+  const int lo = max(0, p_first - window + 1);
+  // this lane's query: pair index 16 * wave + c
+  const int pair = 16 * wave + c;
+  const bool qok = pair < nq * nh;
+  const int tq = qok ? pair / nh : 0, hh = qok ? pair - (pair / nh) * nh : 0;
+  const long row = r0 + t0 + tq;
+  const int h = h0 + hh;
+  const int pq = qok ? pos[row] : -1;
+  const bool wave_live = 16 * wave < nq * nh;
+
+  bf16x8 qf[KSM];
+#pragma unroll
+  for (int ks = 0; ks < KSM; ++ks) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int d = 32 * ks + 8 * g + e;
+      float v = 0.f;
+      if (qok && d < D) v = d < R ? (float)q_lat[(row * H + h) * R + d] : (float)q_rot[(row * H + h) * Dr + d - R];
+      qf[ks][e] = (bf16)v;
+    }
+  }
+  f32x4 o[NTM];
+#pragma unroll
+  for (int nt = 0; nt < NTM; ++nt) o[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  // zero the padding columns / rows once: staging below only writes real elements of staged rows
+  for (int e = threadIdx.x; e < MKT * ldk; e += 256) kt_lds[e] = (bf16)0.f;
+  for (int e = threadIdx.x; e < NT * 16 * MLDV; e += 256) vt_lds[e] = (bf16)0.f;
+
+  for (int k0 = (lo / MKT) * MKT; k0 <= p_last; k0 += MKT) {
+    __syncthreads();
+    const int rows = min(MKT, p_last + 1 - k0);
+    {
+      const long base = ((long)bt[(long)s * btw + k0 / PAGE] * PAGE + (k0 % PAGE)) * D;
+      if ((D & 7) == 0) {                    // rows are whole 16-byte pieces: vector loads and stores
+        const int d8 = D >> 3;
+        for (int e = threadIdx.x; e < MKT * d8; e += 256) {
+          const int j = e / d8, d = (e - j * d8) * 8;
+          bf16x8 v;
+          if (j < rows) v = *reinterpret_cast<const bf16x8*>(cache + base + (long)j * D + d);
+          else
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = (bf16)0.f;
+          *reinterpret_cast<bf16x8*>(kt_lds + j * ldk + d) = v;
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (d + i < R) vt_lds[(d + i) * MLDV + j] = v[i];
+        }
+      } else {
+        for (int e = threadIdx.x; e < MKT * D; e += 256) {
+          const int j = e / D, d = e - j * D;
+          const bf16 v = j < rows ? cache[base + e] : (bf16)0.f;
+          kt_lds[j * ldk + d] = v;
+          if (d < R) vt_lds[d * MLDV + j] = v;
+        }
+      }
+    }
+    __syncthreads();
+    if (!wave_live) continue;
+    // S^T for the two 16-key halves
+    f32x4 st[2];
+    float sc[2][4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {
+      st[kh] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16* kr = kt_lds + (16 * kh + c) * ldk + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < KSM; ++ks)
+        if (ks < KS) st[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(kr + 32 * ks), qf[ks], st[kh], 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = k0 + 16 * kh + 4 * g + i;
+        const bool vis = j <= pq && j > pq - window;
+        sc[kh][i] = vis ? st[kh][i] * scale : -INFINITY;
+        tmax = fmaxf(tmax, sc[kh][i]);
+      }
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float mn = fmaxf(m, tmax);
+    const float corr = (m == -INFINITY) ? 0.f : expf(m - mn);
+    bf16x8 pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = sc[kh][i] == -INFINITY ? 0.f : expf(sc[kh][i] - mn);
+        psum += p;
+        pb[4 * kh + i] = (bf16)p;
+      }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = mn;
+#pragma unroll
+    for (int nt = 0; nt < NTM; ++nt) {
+      if (nt < NT) {
+        const bf16* vr = vt_lds + (16 * nt + c) * MLDV + 4 * g;
+        const bf16x4 a0 = *reinterpret_cast<const bf16x4*>(vr), a1 = *reinterpret_cast<const bf16x4*>(vr + 16);
+        bf16x8 a;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          a[i] = a0[i];
+          a[4 + i] = a1[i];
+        }
+        o[nt] *= corr;
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[nt], 0, 0, 0);
+      }
+    }
+  }
+  if (!qok) return;
+  float gsc = 1.0f / l;
+  if (gate != nullptr) gsc *= mx_sigmoid((float)gate[row * sgate + h]);
+  bf16* dst = out + (row * H + h) * R;
+#pragma unroll
+  for (int nt = 0; nt < NTM; ++nt) {
+    if (nt < NT) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * nt + 4 * g + i;
+        if (r < R) dst[r] = (bf16)(o[nt][i] * gsc);
+      }
+    }
+  }
+}
+
 }  // namespace
+
+// MX_ATTEND_MFMA=0 keeps every call on the f32-lane kernel (A/B and debugging)
+static bool mx_use_mfma() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("MX_ATTEND_MFMA");
+    v = (e != nullptr && e[0] == '0') ? 0 : 1;
+  }
+  return v == 1;
+}
 
 // kv [T, R+Dr] slice (row stride skv); q [T, ...] with head h's rotated part at h*q_head_stride+q_rot_off
 // (row stride sq); q_rot out [T, H, Dr]; cache [pages*64, R+Dr]; all of storage type dt
@@ -217,6 +394,23 @@ MX_API int mx_latent_attend(const void* q_lat, const void* q_rot, const void* ca
   if (S <= 0 || max_len <= 0) return 0;
   if (R > 64 * ATT_RPL) return (int)hipErrorInvalidValue;
   const int D = R + Dr;
+  if (dt == 0 && D <= 320 && R <= 256 && mx_use_mfma()) {
+    // matrix-core form: 64 (row, head) pairs per block
+    const int HB = H < 64 ? H : 64;
+    const int QT = max_len == 1 ? 1 : (64 / HB > 0 ? 64 / HB : 1);
+    const int KS = (D + 31) / 32, NT = (R + 15) / 16;
+    const size_t lds = ((size_t)MKT * (KS * 32 + 8) + (size_t)NT * 16 * MLDV) * sizeof(bf16);
+    dim3 grid((max_len + QT - 1) / QT, (H + HB - 1) / HB, S);
+    if (D <= 128 && R <= 128)
+      latent_attend_mfma_kernel<4, 8><<<grid, 256, lds, st>>>(
+          (const bf16*)q_lat, (const bf16*)q_rot, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate,
+          window, scale, (bf16*)out, H, R, Dr, QT, HB);
+    else
+      latent_attend_mfma_kernel<10, 16><<<grid, 256, lds, st>>>(
+          (const bf16*)q_lat, (const bf16*)q_rot, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate,
+          window, scale, (bf16*)out, H, R, Dr, QT, HB);
+    MX_RETURN_LAUNCH();
+  }
   const int esz = dt == 1 ? 4 : 2;
   // key row stride: odd in 4-byte words
   int ldk = D;

@@ -89,29 +89,45 @@ __global__ void conv_state_kernel(const T* __restrict__ in, long si, float* __re
   }
 }
 
-// Sequential scan.  grid (ceil(P/PT), H, S), block PT * NS threads: thread (p, ns) keeps the state
-// entries S[p][ns + NS*i] in registers; the NS partial sums of y_t[p] are reduced inside the wave.
-// The rows of a chunk of TB tokens (B_t, C_t, the block's x_t, dt and the decay) are staged in LDS;
-// the next chunk's rows are fetched into registers while the current chunk's TB dependent steps
-// run, so the recurrence never waits on HBM.
+// Sequential scan.  grid (ceil(P/PT), H, S), block PT * NS threads: thread (p, ns) keeps the NI
+// consecutive state entries S[p][ns*NI .. ns*NI+NI-1] in registers (a wave's state loads and stores
+// are contiguous runs of the slot's [P][N] record); the NS partial sums of y_t[p] are reduced
+// inside the 16-lane row with DPP swaps.  N is padded to 16 * NI with zeros (B, C and the state
+// entries past N stay 0), so the per-token loop has no bounds checks.  The rows of a chunk of TB
+// tokens (B_t | C_t, the block's x_t, dt and the decay) are staged in LDS; the next chunk's rows
+// are fetched into registers -- unconditional, clamped loads, issued back to back -- before the
+// current chunk's TB dependent steps run, so the recurrence never waits on HBM.
 constexpr int SCAN_NS = 16;       // lanes sharing one value channel
 constexpr int SCAN_PT = 16;       // value channels per block (256 threads)
-constexpr int SCAN_NI = 16;       // state entries per lane: N <= 256
-constexpr int SCAN_PF = 36;       // prefetch registers per thread: TB * (2N + PT + 2) <= 256 * SCAN_PF
+constexpr int SCAN_PF = 36;       // prefetch registers per thread: TB * 2N <= 256 * SCAN_PF
+constexpr int SCAN_NT = SCAN_PT * SCAN_NS;
 
-template <typename TD>
-__global__ void __launch_bounds__(SCAN_PT * SCAN_NS)
+// sum over the 16 lanes of a DPP row, result in every lane: xor 1, xor 2 (quad permutes), then the
+// mirrored 8-lane and 16-lane halves
+__device__ __forceinline__ float row_sum16(float v) {
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));   // row_mirror
+  return v;
+}
+
+template <typename TD, int NI>
+__global__ void __launch_bounds__(SCAN_NT)
 ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_raw, long sdt,
                 const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dp,
                 float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slot,
                 const int* __restrict__ pos, float* __restrict__ y, int H, int P, int N, int G, int TB) {
-  extern __shared__ float rows[];            // [TB][RW]
+  extern __shared__ __align__(16) float rows[];   // [TB][RW]: B[NP] | C[NP] | x[PT] | dt | decay | pad
+  constexpr int NP = SCAN_NS * NI;                // padded state size
+  constexpr int RW = 2 * NP + SCAN_PT + 4;
   const int s = blockIdx.z;
   const int sl = slot[s];
   if (sl < 0) return;
   const int h = blockIdx.y;
-  const int ns = threadIdx.x % SCAN_NS;
-  const int pl = threadIdx.x / SCAN_NS;
+  const int tid = threadIdx.x;
+  const int ns = tid % SCAN_NS;
+  const int pl = tid / SCAN_NS;
   const int p0 = blockIdx.x * SCAN_PT;
   const int p = p0 + pl;
   const bool live = p < P;
@@ -121,77 +137,130 @@ ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_ra
   const int g = h / (H / G);
   const bool fresh = pos[r0] == 0;
   const int inner = H * P;
-  const int RW = 2 * N + SCAN_PT + 2;
+  const int W2 = 2 * N;
+  const int kb = ns * NI;                    // this lane's first state entry
+  const bool vec = (NI % 4 == 0) && N == NP; // 16-byte state and LDS accesses
   float* sp = state + (((long)sl * H + h) * P + pc) * N;
-  float S[SCAN_NI];
+  float S[NI];
+  if (vec) {
 #pragma unroll
-  for (int i = 0; i < SCAN_NI; ++i) {
-    const int k = ns + SCAN_NS * i;
-    S[i] = (!fresh && k < N) ? sp[k] : 0.f;
+    for (int i = 0; i < NI; i += 4) {
+      const float4 v = fresh ? float4{0.f, 0.f, 0.f, 0.f} : *reinterpret_cast<const float4*>(sp + kb + i);
+      S[i] = v.x;
+      S[i + 1 < NI ? i + 1 : i] = v.y;
+      S[i + 2 < NI ? i + 2 : i] = v.z;
+      S[i + 3 < NI ? i + 3 : i] = v.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) S[i] = (!fresh && kb + i < N) ? sp[kb + i] : 0.f;
   }
   const float A = -expf(A_log[h]);
   const float bias = dt_bias[h], Dh = Dp[h];
-  float pf[SCAN_PF];
+  // B_t | C_t of group g are 2N floats that are contiguous when G == 1, two runs otherwise
+  const float* ub = u + inner + g * N;
+  const long c_off = (long)(G - 1) * N;      // extra offset of the C run (col >= N)
+  // per-thread walk over the chunk's TB x 2N elements without divisions
+  const int step_t = SCAN_NT / W2, step_c = SCAN_NT % W2;
+  const int tt0 = tid / W2, col0 = tid % W2;
+  float pf[SCAN_PF], pfx[2], pfd = 0.f;
 
-  auto fetch = [&](int c0) {                 // rows c0 .. c0+TB-1 of the segment -> pf
-    const int cnt = min(TB, n - c0) * RW;
+  auto fetch = [&](int c0) {                 // rows c0 .. c0+TB-1 of the segment -> registers
+    const int last = n - 1 - c0;             // rows past the segment re-read its last row (never used)
+    int tt = tt0, col = col0;
 #pragma unroll
     for (int j = 0; j < SCAN_PF; ++j) {
-      const int e = threadIdx.x + j * (SCAN_PT * SCAN_NS);
-      float v = 0.f;
-      if (e < cnt) {
-        const int tt = e / RW, col = e - tt * RW;
-        const long r = r0 + c0 + tt;
-        const float* ur = u + r * C;
-        if (col < N) v = ur[inner + g * N + col];
-        else if (col < 2 * N) v = ur[inner + G * N + g * N + (col - N)];
-        else if (col < 2 * N + SCAN_PT) {
-          const int pp = p0 + col - 2 * N;
-          v = pp < P ? ur[h * P + pp] : 0.f;
-        } else {
-          const float dt = mx_softplus(ldf(dt_raw + r * sdt + h) + bias);
-          v = col == 2 * N + SCAN_PT ? dt : expf(A * dt);
-        }
+      const long r = r0 + c0 + min(tt, last);
+      pf[j] = ub[r * C + col + (col >= N ? c_off : 0)];
+      col += step_c;
+      tt += step_t;
+      if (col >= W2) {
+        col -= W2;
+        ++tt;
       }
-      pf[j] = v;
     }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = tid + j * SCAN_NT;       // (token, channel) of the block's x
+      const int tx = e / SCAN_PT, px = p0 + e % SCAN_PT;
+      pfx[j] = u[(r0 + c0 + min(tx, last)) * C + h * P + min(px, P - 1)];
+    }
+    pfd = ldf(dt_raw + (r0 + c0 + min(tid, last)) * sdt + h);
   };
 
+  if (N != NP)                               // the padding columns of B and C stay zero
+    for (int e = tid; e < TB * RW; e += SCAN_NT) rows[e] = 0.f;
   fetch(0);
   for (int c0 = 0; c0 < n; c0 += TB) {
     const int m = min(TB, n - c0);
     __syncthreads();                         // the previous chunk's readers are done
+    {
+      int tt = tt0, col = col0;
 #pragma unroll
-    for (int j = 0; j < SCAN_PF; ++j) {
-      const int e = threadIdx.x + j * (SCAN_PT * SCAN_NS);
-      if (e < m * RW) rows[e] = pf[j];
-    }
-    __syncthreads();
-    if (c0 + TB < n) fetch(c0 + TB);
-    for (int t = 0; t < m; ++t) {
-      const float* row = rows + t * RW;
-      const float x = row[2 * N + pl];
-      const float dt = row[2 * N + SCAN_PT], a = row[2 * N + SCAN_PT + 1];
-      const float dx = dt * x;
-      float acc = 0.f;
-#pragma unroll
-      for (int i = 0; i < SCAN_NI; ++i) {
-        const int k = ns + SCAN_NS * i;
-        if (k < N) {
-          S[i] = a * S[i] + dx * row[k];
-          acc += S[i] * row[N + k];
+      for (int j = 0; j < SCAN_PF; ++j) {
+        if (tt < TB) rows[tt * RW + (col >= N ? col - N + NP : col)] = pf[j];
+        col += step_c;
+        tt += step_t;
+        if (col >= W2) {
+          col -= W2;
+          ++tt;
         }
       }
 #pragma unroll
-      for (int o = SCAN_NS / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+      for (int j = 0; j < 2; ++j) {
+        const int e = tid + j * SCAN_NT;
+        if (e / SCAN_PT < TB) rows[(e / SCAN_PT) * RW + 2 * NP + e % SCAN_PT] = pfx[j];
+      }
+      if (tid < TB) {
+        const float dt = mx_softplus(pfd + bias);
+        rows[tid * RW + 2 * NP + SCAN_PT] = dt;
+        rows[tid * RW + 2 * NP + SCAN_PT + 1] = expf(A * dt);
+      }
+    }
+    __syncthreads();
+    if (c0 + TB < n) fetch(c0 + TB);
+#pragma unroll 2
+    for (int t = 0; t < m; ++t) {
+      const float* row = rows + t * RW;
+      const float x = row[2 * NP + pl];
+      const float2 da = *reinterpret_cast<const float2*>(row + 2 * NP + SCAN_PT);
+      const float dx = da.x * x;
+      float Bv[NI], Cv[NI];
+      if (NI % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < NI; i += 4) {
+          const float4 b4 = *reinterpret_cast<const float4*>(row + kb + i);
+          const float4 c4 = *reinterpret_cast<const float4*>(row + NP + kb + i);
+          Bv[i] = b4.x; Bv[i + 1 < NI ? i + 1 : i] = b4.y; Bv[i + 2 < NI ? i + 2 : i] = b4.z; Bv[i + 3 < NI ? i + 3 : i] = b4.w;
+          Cv[i] = c4.x; Cv[i + 1 < NI ? i + 1 : i] = c4.y; Cv[i + 2 < NI ? i + 2 : i] = c4.z; Cv[i + 3 < NI ? i + 3 : i] = c4.w;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          Bv[i] = row[kb + i];
+          Cv[i] = row[NP + kb + i];
+        }
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        S[i] = da.y * S[i] + dx * Bv[i];
+        acc += S[i] * Cv[i];
+      }
+      acc = row_sum16(acc);
       if (ns == 0 && live) y[(long)(r0 + c0 + t) * inner + h * P + p] = acc + Dh * x;
     }
   }
   if (live) {
+    if (vec) {
 #pragma unroll
-    for (int i = 0; i < SCAN_NI; ++i) {
-      const int k = ns + SCAN_NS * i;
-      if (k < N) sp[k] = S[i];
+      for (int i = 0; i < NI; i += 4)
+        *reinterpret_cast<float4*>(sp + kb + i) =
+            float4{S[i], S[i + 1 < NI ? i + 1 : i], S[i + 2 < NI ? i + 2 : i], S[i + 3 < NI ? i + 3 : i]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        if (kb + i < N) sp[kb + i] = S[i];
     }
   }
 }
@@ -220,14 +289,23 @@ MX_API int mx_ssm_scan(const float* u, int C, const void* dt_raw, long sdt, int 
                        const float* A_log, const float* D, float* state, const int* cu, const int* slot,
                        const int* pos, float* y, int S, int H, int P, int N, int G, hipStream_t st) {
   if (S <= 0) return 0;
-  if (N > SCAN_NS * SCAN_NI || G < 1 || H % G) return (int)hipErrorInvalidValue;
+  if (N > SCAN_NS * 16 || G < 1 || H % G) return (int)hipErrorInvalidValue;
   dim3 grid((P + SCAN_PT - 1) / SCAN_PT, H, S);
-  const int RW = 2 * N + SCAN_PT + 2;
-  int TB = (SCAN_PT * SCAN_NS * SCAN_PF) / RW;
+  int TB = (SCAN_NT * SCAN_PF) / (2 * N);
   TB = TB > 32 ? 32 : TB;
   if (TB < 1) return (int)hipErrorInvalidValue;
-  const size_t lds = (size_t)TB * RW * sizeof(float);
-  MX_DISPATCH(dt_code, TT, ssm_scan_kernel<TT><<<grid, SCAN_PT * SCAN_NS, lds, st>>>(
-      u, C, (const TT*)dt_raw, sdt, dt_bias, A_log, D, state, cu, slot, pos, y, H, P, N, G, TB));
+  const int need = (N + SCAN_NS - 1) / SCAN_NS;         // state entries per lane, rounded up to 1, 2, 4, 8, 16
+#define MX_SCAN(NI)                                                                                          \
+  do {                                                                                                       \
+    const size_t lds = (size_t)TB * (2 * SCAN_NS * NI + SCAN_PT + 4) * sizeof(float);                        \
+    MX_DISPATCH(dt_code, TT, ssm_scan_kernel<TT, NI><<<grid, SCAN_NT, lds, st>>>(                            \
+        u, C, (const TT*)dt_raw, sdt, dt_bias, A_log, D, state, cu, slot, pos, y, H, P, N, G, TB));         \
+  } while (0)
+  if (need <= 1) MX_SCAN(1);
+  else if (need <= 2) MX_SCAN(2);
+  else if (need <= 4) MX_SCAN(4);
+  else if (need <= 8) MX_SCAN(8);
+  else MX_SCAN(16);
+#undef MX_SCAN
   MX_RETURN_LAUNCH();
 }

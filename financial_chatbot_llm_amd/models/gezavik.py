@@ -105,31 +105,33 @@ class GezavikModel:
         return s
 
     @staticmethod
-    def _random(name: str, shape, seed: int) -> torch.Tensor:
-        g = torch.Generator().manual_seed(param_seed(seed, name))
+    def _random(name: str, shape, seed: int, device="cpu") -> torch.Tensor:
+        g = torch.Generator(device=device).manual_seed(param_seed(seed, name))
+        randn = lambda: torch.randn(shape, generator=g, device=device)  # noqa: E731
+        rand = lambda: torch.rand(shape, generator=g, device=device)  # noqa: E731
         leaf = name.rsplit(".", 1)[-1]
         if leaf in ("norm1", "norm") and len(shape) == 1:
-            return 1.0 + 0.1 * torch.randn(shape, generator=g)
+            return 1.0 + 0.1 * randn()
         if leaf == "A_log":
-            return torch.log(1.0 + 7.0 * torch.rand(shape, generator=g))
+            return torch.log(1.0 + 7.0 * rand())
         if leaf == "dt_bias":      # softplus^-1 of step sizes in [0.01, 0.2]
-            dt = torch.exp(torch.rand(shape, generator=g) * (math.log(0.2) - math.log(0.01)) + math.log(0.01))
+            dt = torch.exp(rand() * (math.log(0.2) - math.log(0.01)) + math.log(0.01))
             return dt + torch.log(-torch.expm1(-dt))
         if leaf == "D":
-            return 1.0 + 0.2 * torch.randn(shape, generator=g)
+            return 1.0 + 0.2 * randn()
         if leaf == "correction":
-            return 0.05 * torch.randn(shape, generator=g)
+            return 0.05 * randn()
         if leaf == "b":
-            return 0.1 * torch.randn(shape, generator=g)
+            return 0.1 * randn()
         if leaf == "conv":
-            return torch.randn(shape, generator=g) * shape[1] ** -0.5
+            return randn() * shape[1] ** -0.5
         if leaf == "embed":
-            return torch.randn(shape, generator=g)
-        return torch.randn(shape, generator=g) * shape[-1] ** -0.5
+            return randn()
+        return randn() * shape[-1] ** -0.5
 
     def init_random(self, seed: int = 0, std: float = 0.02) -> "GezavikModel":
         """Deterministic per-name weights, rounded to bf16 as a checkpoint would hold them."""
-        sd = {n: self._random(n, s, seed).to(torch.bfloat16) for n, s in self.full_shapes().items()}
+        sd = {n: self._random(n, s, seed, self.device).to(torch.bfloat16) for n, s in self.full_shapes().items()}
         return self.load_state(sd)
 
     def load_state(self, sd: Dict[str, torch.Tensor]) -> "GezavikModel":
