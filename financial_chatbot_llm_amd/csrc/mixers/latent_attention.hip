@@ -216,7 +216,8 @@ __global__ void __launch_bounds__(256)
 latent_attend_mfma_kernel(const bf16* __restrict__ q_lat, const bf16* __restrict__ q_rot,
                           const bf16* __restrict__ cache, const int* __restrict__ cu, const int* __restrict__ pos,
                           const int* __restrict__ bt, int btw, const bf16* __restrict__ gate, long sgate, int window,
-                          float scale, bf16* __restrict__ out, int H, int R, int Dr, int QT, int HB) {
+                          float scale, bf16* __restrict__ out, int H, int R, int Dr, int QT, int HB, int nsplit,
+                          float* __restrict__ ws) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int D = R + Dr;
   const int KS = (D + 31) / 32, NT = (R + 15) / 16;
@@ -225,7 +226,9 @@ latent_attend_mfma_kernel(const bf16* __restrict__ q_lat, const bf16* __restrict
   bf16* vt_lds = kt_lds + MKT * ldk;                            // [NT*16][MLDV]
   const int s = blockIdx.z;
   const int r0 = cu[s], n = cu[s + 1] - r0;
-  const int t0 = blockIdx.x * QT;
+  // nsplit > 1 (single-row segments): blockIdx.x is the part of the key range this block walks
+  const int split = nsplit > 1 ? blockIdx.x : 0;
+  const int t0 = nsplit > 1 ? 0 : blockIdx.x * QT;
   if (t0 >= n) return;
   const int nq = min(QT, n - t0);
   const int h0 = blockIdx.y * HB;
@@ -262,7 +265,14 @@ latent_attend_mfma_kernel(const bf16* __restrict__ q_lat, const bf16* __restrict
   for (int e = threadIdx.x; e < MKT * ldk; e += 256) kt_lds[e] = (bf16)0.f;
   for (int e = threadIdx.x; e < NT * 16 * MLDV; e += 256) vt_lds[e] = (bf16)0.f;
 
-  for (int k0 = (lo / MKT) * MKT; k0 <= p_last; k0 += MKT) {
+  int k_begin = (lo / MKT) * MKT, k_end = p_last;     // first tile start, last key
+  if (nsplit > 1) {
+    const int tiles = (p_last - k_begin) / MKT + 1;
+    const int per = (tiles + nsplit - 1) / nsplit;
+    k_begin += split * per * MKT;
+    k_end = min(p_last, k_begin + per * MKT - 1);
+  }
+  for (int k0 = k_begin; k0 <= k_end; k0 += MKT) {
     __syncthreads();
     const int rows = min(MKT, p_last + 1 - k0);
     {
@@ -346,6 +356,22 @@ latent_attend_mfma_kernel(const bf16* __restrict__ q_lat, const bf16* __restrict
     }
   }
   if (!qok) return;
+  if (nsplit > 1) {                          // unnormalised part: o | m | l, merged by latent_merge_kernel
+    float* w = ws + ((row * H + h) * nsplit + split) * (long)(R + 2);
+#pragma unroll
+    for (int nt = 0; nt < NTM; ++nt)
+      if (nt < NT)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = 16 * nt + 4 * g + i;
+          if (r < R) w[r] = o[nt][i];
+        }
+    if (g == 0) {
+      w[R] = m;
+      w[R + 1] = l;
+    }
+    return;
+  }
   float gsc = 1.0f / l;
   if (gate != nullptr) gsc *= mx_sigmoid((float)gate[row * sgate + h]);
   bf16* dst = out + (row * H + h) * R;
@@ -358,6 +384,31 @@ latent_attend_mfma_kernel(const bf16* __restrict__ q_lat, const bf16* __restrict
         if (r < R) dst[r] = (bf16)(o[nt][i] * gsc);
       }
     }
+  }
+}
+
+// grid (rows, H): combine the nsplit parts of one (row, head)
+__global__ void latent_merge_kernel(const float* __restrict__ ws, const bf16* __restrict__ gate, long sgate,
+                                    bf16* __restrict__ out, int H, int R, int nsplit) {
+  const long row = blockIdx.x;
+  const int h = blockIdx.y;
+  const float* w = ws + (row * H + h) * nsplit * (long)(R + 2);
+  float M = -INFINITY;
+  for (int i = 0; i < nsplit; ++i) M = fmaxf(M, w[i * (R + 2) + R]);
+  float L = 0.f;
+  for (int i = 0; i < nsplit; ++i) {
+    const float mi = w[i * (R + 2) + R];
+    if (mi != -INFINITY) L += w[i * (R + 2) + R + 1] * expf(mi - M);
+  }
+  float gsc = 1.0f / L;
+  if (gate != nullptr) gsc *= mx_sigmoid((float)gate[row * sgate + h]);
+  for (int r = threadIdx.x; r < R; r += blockDim.x) {
+    float a = 0.f;
+    for (int i = 0; i < nsplit; ++i) {
+      const float mi = w[i * (R + 2) + R];
+      if (mi != -INFINITY) a += w[i * (R + 2) + r] * expf(mi - M);
+    }
+    out[(row * H + h) * R + r] = (bf16)(a * gsc);
   }
 }
 
@@ -388,9 +439,12 @@ MX_API int mx_latent_prep(const void* kv, long skv, const float* norm_w, float e
 
 // q_lat [T, H, R], q_rot [T, H, Dr], out [T, H, R] contiguous; cu [S+1] row bounds of the segments,
 // pos [T] positions, bt [S, btw] page tables; gate [T, >=H] slice (row stride sgate) or null.
+// nsplit > 1 with a workspace ws (f32 [T, H, nsplit, R + 2]) and single-row segments: the key range of
+// each row is walked by nsplit blocks and merged (bf16 matrix-core form only; ignored otherwise).
 MX_API int mx_latent_attend(const void* q_lat, const void* q_rot, const void* cache, const int* cu, const int* pos,
                             const int* bt, int btw, const void* gate, long sgate, int window, float scale,
-                            void* out, int dt, int S, int max_len, int H, int R, int Dr, hipStream_t st) {
+                            void* out, int dt, int S, int max_len, int H, int R, int Dr, int nsplit, float* ws,
+                            hipStream_t st) {
   if (S <= 0 || max_len <= 0) return 0;
   if (R > 64 * ATT_RPL) return (int)hipErrorInvalidValue;
   const int D = R + Dr;
@@ -400,15 +454,20 @@ MX_API int mx_latent_attend(const void* q_lat, const void* q_rot, const void* ca
     const int QT = max_len == 1 ? 1 : (64 / HB > 0 ? 64 / HB : 1);
     const int KS = (D + 31) / 32, NT = (R + 15) / 16;
     const size_t lds = ((size_t)MKT * (KS * 32 + 8) + (size_t)NT * 16 * MLDV) * sizeof(bf16);
-    dim3 grid((max_len + QT - 1) / QT, (H + HB - 1) / HB, S);
+    if (max_len != 1 || ws == nullptr || nsplit < 1) nsplit = 1;
+    dim3 grid(nsplit > 1 ? nsplit : (max_len + QT - 1) / QT, (H + HB - 1) / HB, S);
     if (D <= 128 && R <= 128)
       latent_attend_mfma_kernel<4, 8><<<grid, 256, lds, st>>>(
           (const bf16*)q_lat, (const bf16*)q_rot, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate,
-          window, scale, (bf16*)out, H, R, Dr, QT, HB);
+          window, scale, (bf16*)out, H, R, Dr, QT, HB, nsplit, ws);
     else
       latent_attend_mfma_kernel<10, 16><<<grid, 256, lds, st>>>(
           (const bf16*)q_lat, (const bf16*)q_rot, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate,
-          window, scale, (bf16*)out, H, R, Dr, QT, HB);
+          window, scale, (bf16*)out, H, R, Dr, QT, HB, nsplit, ws);
+    if (nsplit > 1) {
+      dim3 g2(S, H);           // single-row segments: row index == segment index
+      latent_merge_kernel<<<g2, R >= 128 ? 128 : 64, 0, st>>>(ws, (const bf16*)gate, sgate, (bf16*)out, H, R, nsplit);
+    }
     MX_RETURN_LAUNCH();
   }
   const int esz = dt == 1 ? 4 : 2;

@@ -188,6 +188,52 @@ ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_ra
     pfd = ldf(dt_raw + (r0 + c0 + min(tid, last)) * sdt + h);
   };
 
+  if (n == 1) {
+    // a decoded token: no staging -- every lane reads its own B / C entries and the row's scalars
+    const float* ur = u + (long)r0 * C;
+    const float dt = mx_softplus(ldf(dt_raw + (long)r0 * sdt + h) + bias);
+    const float a = expf(A * dt);
+    const float x = ur[h * P + pc];
+    const float dx = dt * x;
+    const float* Br = ub + (long)r0 * C + kb;
+    const float* Cr = Br + N + c_off;
+    float acc0 = 0.f, acc1 = 0.f;
+    if (vec && (inner & 3) == 0 && (C & 3) == 0) {      // the row's B / C runs are 16-byte aligned too
+#pragma unroll
+      for (int i = 0; i < NI; i += 4) {
+        const float4 b4 = *reinterpret_cast<const float4*>(Br + i), c4 = *reinterpret_cast<const float4*>(Cr + i);
+        const float bb[4] = {b4.x, b4.y, b4.z, b4.w}, cc[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int k = i + j < NI ? i + j : i;
+          S[k] = a * S[k] + dx * bb[j];
+          if (j & 1) acc1 += S[k] * cc[j]; else acc0 += S[k] * cc[j];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        if (kb + i < N) {
+          S[i] = a * S[i] + dx * Br[i];
+          acc0 += S[i] * Cr[i];
+        }
+    }
+    const float acc = row_sum16(acc0 + acc1);
+    if (live) {
+      if (ns == 0) y[(long)r0 * inner + h * P + p] = acc + Dh * x;
+      if (vec) {
+#pragma unroll
+        for (int i = 0; i < NI; i += 4)
+          *reinterpret_cast<float4*>(sp + kb + i) =
+              float4{S[i], S[i + 1 < NI ? i + 1 : i], S[i + 2 < NI ? i + 2 : i], S[i + 3 < NI ? i + 3 : i]};
+      } else {
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+          if (kb + i < N) sp[kb + i] = S[i];
+      }
+    }
+    return;
+  }
   if (N != NP)                               // the padding columns of B and C stay zero
     for (int e = tid; e < TB * RW; e += SCAN_NT) rows[e] = 0.f;
   fetch(0);
@@ -241,13 +287,13 @@ ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_ra
           Cv[i] = row[NP + kb + i];
         }
       }
-      float acc = 0.f;
+      float acc = 0.f, acc1 = 0.f;
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         S[i] = da.y * S[i] + dx * Bv[i];
-        acc += S[i] * Cv[i];
+        if (i & 1) acc1 += S[i] * Cv[i]; else acc += S[i] * Cv[i];
       }
-      acc = row_sum16(acc);
+      acc = row_sum16(acc + acc1);
       if (ns == 0 && live) y[(long)(r0 + c0 + t) * inner + h * P + p] = acc + Dh * x;
     }
   }

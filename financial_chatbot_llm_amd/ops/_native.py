@@ -97,7 +97,7 @@ _MIXER_SIGS = {
     "mx_latent_prep": [P, c_long, P, c_float, P, c_int, P, P, P, P, c_long, c_int, c_int, P, c_int, c_int, c_int,
                        c_int, c_int, P],
     "mx_latent_attend": [P, P, P, P, P, P, c_int, P, c_long, c_int, c_float, P, c_int, c_int, c_int, c_int, c_int,
-                         c_int, P],
+                         c_int, c_int, P, P],
 }
 _MIXER_LIB: Optional[ctypes.CDLL] = None
 

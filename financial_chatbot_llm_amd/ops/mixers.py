@@ -309,10 +309,18 @@ def latent_attend(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor,
     if N.use_native(q_lat):
         assert q_lat.is_contiguous() and q_rot.is_contiguous() and bt.is_contiguous()
         out = torch.empty((T, H, R), dtype=q_lat.dtype, device=q_lat.device)
+        # decode-size steps (one row per segment) walk each row's keys with several blocks so that a
+        # small batch still fills the chip; the split depends only on static sizes (graph-safe)
+        nsplit, ws = 1, None
+        if max_len == 1 and q_lat.dtype == torch.bfloat16:
+            tiles = (min(window, bt.shape[1] * PAGE) + 31) // 32 + 1
+            nsplit = max(1, min(16, tiles // 2, 1024 // max(S * ((H + 63) // 64), 1)))
+            if nsplit > 1:
+                ws = torch.empty((T, H, nsplit, R + 2), dtype=torch.float32, device=q_lat.device)
         N.mcall("mx_latent_attend", N.ptr(q_lat), N.ptr(q_rot), N.ptr(cache), N.ptr(cu), N.ptr(pos), N.ptr(bt),
                 bt.shape[1], N.ptr(_rows(gate)) if gate is not None else None,
                 gate.stride(0) if gate is not None else 0, int(min(window, 1 << 30)), float(scale), N.ptr(out),
-                _dt(q_lat), S, int(max_len), H, R, Dr, N.stream())
+                _dt(q_lat), S, int(max_len), H, R, Dr, nsplit, N.ptr(ws), N.stream())
         return out
     out = torch.zeros((T, H, R), dtype=torch.float32)
     rows = cache.view(-1, R + Dr).float()

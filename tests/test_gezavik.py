@@ -281,6 +281,27 @@ def test_far_key_in_a_long_prompt_chunk(device):
         assert bool((out[:, :, 1] > 25.0).all()) == hit
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("window", [1 << 30, 150])
+def test_decode_rows_split_over_keys(window):
+    """Single decoded rows of bf16 models walk their keys with several blocks whose parts are merged:
+    rows at unequal depths, pages in scrambled order, against the one-pass CPU form."""
+    H, R, Dr, pages = 5, 48, 16, 12
+    g = torch.Generator().manual_seed(9)
+    cache = torch.randn(pages * 64, R + Dr, generator=g).bfloat16()
+    depths = [700, 33, 64, 301, 1]
+    bt = torch.stack([torch.randperm(pages, generator=g) for _ in depths]).to(torch.int32)
+    pos = torch.tensor([d - 1 for d in depths], dtype=torch.int32)
+    cu = torch.arange(len(depths) + 1, dtype=torch.int32)
+    q = (0.3 * torch.randn(len(depths), H, R, generator=g)).bfloat16()
+    qr = (0.3 * torch.randn(len(depths), H, Dr, generator=g)).bfloat16()
+    gate = torch.randn(len(depths), H, generator=g).bfloat16()
+    want = mx.latent_attend(q, qr, cache, cu, pos, bt, window, 0.2, 1, gate=gate).float()
+    got = mx.latent_attend(q.cuda(), qr.cuda(), cache.cuda(), cu.cuda(), pos.cuda(), bt.cuda(), window, 0.2, 1,
+                           gate=gate.cuda()).float().cpu()
+    assert (got - want).abs().max() < 2e-2
+
+
 # ---------------------------------------------------------------------------------------------------
 # routing
 # ---------------------------------------------------------------------------------------------------
