@@ -212,7 +212,7 @@ constexpr int MKT = 32;             // keys per tile
 constexpr int MLDV = MKT + 8;       // row stride of the transposed value tile
 
 template <int KSM, int NTM>         // up to 32*KSM key dims, 16*NTM value dims
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))   // two blocks per CU: <= 256 registers
 latent_attend_mfma_kernel(const bf16* __restrict__ q_lat, const bf16* __restrict__ q_rot,
                           const bf16* __restrict__ cache, const int* __restrict__ cu, const int* __restrict__ pos,
                           const int* __restrict__ bt, int btw, const bf16* __restrict__ gate, long sgate, int window,
@@ -272,35 +272,66 @@ latent_attend_mfma_kernel(const bf16* __restrict__ q_lat, const bf16* __restrict
     k_begin += split * per * MKT;
     k_end = min(p_last, k_begin + per * MKT - 1);
   }
+  // staging, 16-byte path (rows are whole 16-byte pieces): a work item is a pair of keys x 8 dims --
+  // two row loads, two 16-byte stores into the key tile and eight 4-byte stores (one key pair
+  // each) into the transposed value tile.  The next tile's loads are issued before the current
+  // tile's MFMAs and land in registers while they run.
+  constexpr int MAXIT = 3;                   // 16 pairs * (<= 40 pieces) / 256 threads
+  const bool v16 = (D & 7) == 0;
+  const int d8 = D >> 3;
+  bf16x8 pre[MAXIT][2];
+  auto load_tile = [&](int k0) {
+    const int rows = min(MKT, p_last + 1 - k0);
+    const bf16* src = cache + ((long)bt[(long)s * btw + k0 / PAGE] * PAGE + (k0 % PAGE)) * D;
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int e = min((int)threadIdx.x + 256 * it, 16 * d8 - 1);
+      const int d = (e >> 4) * 8, jp = e & 15;
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int j = 2 * jp + r;
+        bf16x8 v = *reinterpret_cast<const bf16x8*>(src + (long)min(j, rows - 1) * D + d);
+        if (j >= rows)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[i] = (bf16)0.f;
+        pre[it][r] = v;
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int e = threadIdx.x + 256 * it;
+      if (e < 16 * d8) {
+        const int d = (e >> 4) * 8, jp = e & 15;
+        *reinterpret_cast<bf16x8*>(kt_lds + (2 * jp) * ldk + d) = pre[it][0];
+        *reinterpret_cast<bf16x8*>(kt_lds + (2 * jp + 1) * ldk + d) = pre[it][1];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (d + i < R) {
+            typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+            *reinterpret_cast<bf16x2*>(vt_lds + (d + i) * MLDV + 2 * jp) = bf16x2{pre[it][0][i], pre[it][1][i]};
+          }
+      }
+    }
+  };
+  if (v16 && k_begin <= k_end) load_tile(k_begin);
   for (int k0 = k_begin; k0 <= k_end; k0 += MKT) {
     __syncthreads();
     const int rows = min(MKT, p_last + 1 - k0);
-    {
+    if (v16) {
+      store_tile();
+    } else {
       const long base = ((long)bt[(long)s * btw + k0 / PAGE] * PAGE + (k0 % PAGE)) * D;
-      if ((D & 7) == 0) {                    // rows are whole 16-byte pieces: vector loads and stores
-        const int d8 = D >> 3;
-        for (int e = threadIdx.x; e < MKT * d8; e += 256) {
-          const int j = e / d8, d = (e - j * d8) * 8;
-          bf16x8 v;
-          if (j < rows) v = *reinterpret_cast<const bf16x8*>(cache + base + (long)j * D + d);
-          else
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = (bf16)0.f;
-          *reinterpret_cast<bf16x8*>(kt_lds + j * ldk + d) = v;
-#pragma unroll
-          for (int i = 0; i < 8; ++i)
-            if (d + i < R) vt_lds[(d + i) * MLDV + j] = v[i];
-        }
-      } else {
-        for (int e = threadIdx.x; e < MKT * D; e += 256) {
-          const int j = e / D, d = e - j * D;
-          const bf16 v = j < rows ? cache[base + e] : (bf16)0.f;
-          kt_lds[j * ldk + d] = v;
-          if (d < R) vt_lds[d * MLDV + j] = v;
-        }
+      for (int e = threadIdx.x; e < MKT * D; e += 256) {
+        const int j = e / D, d = e - j * D;
+        const bf16 v = j < rows ? cache[base + e] : (bf16)0.f;
+        kt_lds[j * ldk + d] = v;
+        if (d < R) vt_lds[d * MLDV + j] = v;
       }
     }
     __syncthreads();
+    if (v16 && k0 + MKT <= k_end) load_tile(k0 + MKT);
     if (!wave_live) continue;
     // S^T for the two 16-key halves
     f32x4 st[2];

@@ -11,6 +11,8 @@
 //            dt = softplus(dt_raw + dt_bias[h]);  a = exp(-exp(A_log[h]) * dt)
 //            S <- a * S + dt * x_t (outer) B_t;   y_t = S C_t + D[h] * x_t
 //          u rows are laid out [x: H*P | B: G*N | C: G*N].
+#include <type_traits>
+
 #include "mx_common.h"
 
 namespace {
@@ -112,8 +114,9 @@ __device__ __forceinline__ float row_sum16(float v) {
   return v;
 }
 
-template <typename TD, int NI>
-__global__ void __launch_bounds__(SCAN_NT)
+// VEC: B | C rows are fetched and staged as 16-byte pieces (N, H*P and the row stride multiples of 4)
+template <typename TD, int NI, bool VEC>
+__global__ void __launch_bounds__(SCAN_NT) __attribute__((amdgpu_waves_per_eu(NI <= 8 ? 3 : 2)))   // blocks per CU that hide the step latency
 ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_raw, long sdt,
                 const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dp,
                 float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slot,
@@ -160,22 +163,28 @@ ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_ra
   // B_t | C_t of group g are 2N floats that are contiguous when G == 1, two runs otherwise
   const float* ub = u + inner + g * N;
   const long c_off = (long)(G - 1) * N;      // extra offset of the C run (col >= N)
-  // per-thread walk over the chunk's TB x 2N elements without divisions
-  const int step_t = SCAN_NT / W2, step_c = SCAN_NT % W2;
-  const int tt0 = tid / W2, col0 = tid % W2;
-  float pf[SCAN_PF], pfx[2], pfd = 0.f;
+  // per-thread walk over the chunk's TB x 2N elements (in pieces of UW floats) without divisions
+  using U = std::conditional_t<VEC, float4, float>;
+  constexpr int UW = VEC ? 4 : 1, PFN = SCAN_PF / UW;
+  const int W2u = W2 / UW;
+  const int step_t = SCAN_NT / W2u, step_c = SCAN_NT % W2u;
+  const int tt0 = tid / W2u, col0 = tid % W2u;
+  U pf[PFN];
+  float pfx[2], pfd = 0.f;
 
+  // (32-bit element offsets from the block-uniform bases: the launcher checks rows * C < 2^31)
   auto fetch = [&](int c0) {                 // rows c0 .. c0+TB-1 of the segment -> registers
     const int last = n - 1 - c0;             // rows past the segment re-read its last row (never used)
     int tt = tt0, col = col0;
 #pragma unroll
-    for (int j = 0; j < SCAN_PF; ++j) {
-      const long r = r0 + c0 + min(tt, last);
-      pf[j] = ub[r * C + col + (col >= N ? c_off : 0)];
+    for (int j = 0; j < PFN; ++j) {
+      const int r = r0 + c0 + min(tt, last);
+      const int ce = col * UW;
+      pf[j] = *reinterpret_cast<const U*>(ub + (unsigned)(r * C + ce + (ce >= N ? (int)c_off : 0)));
       col += step_c;
       tt += step_t;
-      if (col >= W2) {
-        col -= W2;
+      if (col >= W2u) {
+        col -= W2u;
         ++tt;
       }
     }
@@ -183,7 +192,7 @@ ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_ra
     for (int j = 0; j < 2; ++j) {
       const int e = tid + j * SCAN_NT;       // (token, channel) of the block's x
       const int tx = e / SCAN_PT, px = p0 + e % SCAN_PT;
-      pfx[j] = u[(r0 + c0 + min(tx, last)) * C + h * P + min(px, P - 1)];
+      pfx[j] = u[(unsigned)((r0 + c0 + min(tx, last)) * C + h * P + min(px, P - 1))];
     }
     pfd = ldf(dt_raw + (r0 + c0 + min(tid, last)) * sdt + h);
   };
@@ -243,12 +252,13 @@ ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_ra
     {
       int tt = tt0, col = col0;
 #pragma unroll
-      for (int j = 0; j < SCAN_PF; ++j) {
-        if (tt < TB) rows[tt * RW + (col >= N ? col - N + NP : col)] = pf[j];
+      for (int j = 0; j < PFN; ++j) {
+        const int ce = col * UW;
+        if (tt < TB) *reinterpret_cast<U*>(rows + tt * RW + (ce >= N ? ce - N + NP : ce)) = pf[j];
         col += step_c;
         tt += step_t;
-        if (col >= W2) {
-          col -= W2;
+        if (col >= W2u) {
+          col -= W2u;
           ++tt;
         }
       }
@@ -265,7 +275,6 @@ ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_ra
     }
     __syncthreads();
     if (c0 + TB < n) fetch(c0 + TB);
-#pragma unroll 2
     for (int t = 0; t < m; ++t) {
       const float* row = rows + t * RW;
       const float x = row[2 * NP + pl];
@@ -333,19 +342,26 @@ MX_API int mx_conv_silu(const void* in, long si, int dt, const float* w, const f
 // [slots, H, P, N]; y f32 [rows, H*P]
 MX_API int mx_ssm_scan(const float* u, int C, const void* dt_raw, long sdt, int dt_code, const float* dt_bias,
                        const float* A_log, const float* D, float* state, const int* cu, const int* slot,
-                       const int* pos, float* y, int S, int H, int P, int N, int G, hipStream_t st) {
+                       const int* pos, float* y, int S, int H, int P, int N, int G, int cu_rows_bound,
+                       hipStream_t st) {
   if (S <= 0) return 0;
   if (N > SCAN_NS * 16 || G < 1 || H % G) return (int)hipErrorInvalidValue;
+  if ((long)cu_rows_bound * C >= (1L << 31)) return (int)hipErrorInvalidValue;
   dim3 grid((P + SCAN_PT - 1) / SCAN_PT, H, S);
   int TB = (SCAN_NT * SCAN_PF) / (2 * N);
   TB = TB > 32 ? 32 : TB;
   if (TB < 1) return (int)hipErrorInvalidValue;
+  const bool vecu = (N % 4 == 0) && ((H * P) % 4 == 0) && (C % 4 == 0);
   const int need = (N + SCAN_NS - 1) / SCAN_NS;         // state entries per lane, rounded up to 1, 2, 4, 8, 16
 #define MX_SCAN(NI)                                                                                          \
   do {                                                                                                       \
     const size_t lds = (size_t)TB * (2 * SCAN_NS * NI + SCAN_PT + 4) * sizeof(float);                        \
-    MX_DISPATCH(dt_code, TT, ssm_scan_kernel<TT, NI><<<grid, SCAN_NT, lds, st>>>(                            \
-        u, C, (const TT*)dt_raw, sdt, dt_bias, A_log, D, state, cu, slot, pos, y, H, P, N, G, TB));         \
+    if (vecu)                                                                                                \
+      MX_DISPATCH(dt_code, TT, ssm_scan_kernel<TT, NI, true><<<grid, SCAN_NT, lds, st>>>(                    \
+          u, C, (const TT*)dt_raw, sdt, dt_bias, A_log, D, state, cu, slot, pos, y, H, P, N, G, TB));       \
+    else                                                                                                     \
+      MX_DISPATCH(dt_code, TT, ssm_scan_kernel<TT, NI, false><<<grid, SCAN_NT, lds, st>>>(                   \
+          u, C, (const TT*)dt_raw, sdt, dt_bias, A_log, D, state, cu, slot, pos, y, H, P, N, G, TB));       \
   } while (0)
   if (need <= 1) MX_SCAN(1);
   else if (need <= 2) MX_SCAN(2);

@@ -93,7 +93,7 @@ _MIXER_SIGS = {
     "mx_route_biased": [P, P, c_int, c_int, P, P, c_int, P],
     "mx_moe_combine": [P, P, P, P, P, c_long, P, c_long, c_int, c_int, c_int, P, c_int, c_int, P],
     "mx_conv_silu": [P, c_long, c_int, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, P],
-    "mx_ssm_scan": [P, c_int, P, c_long, c_int, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mx_ssm_scan": [P, c_int, P, c_long, c_int, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mx_latent_prep": [P, c_long, P, c_float, P, c_int, P, P, P, P, c_long, c_int, c_int, P, c_int, c_int, c_int,
                        c_int, c_int, P],
     "mx_latent_attend": [P, P, P, P, P, P, c_int, P, c_long, c_int, c_float, P, c_int, c_int, c_int, c_int, c_int,

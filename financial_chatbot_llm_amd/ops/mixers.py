@@ -224,7 +224,7 @@ def ssm_scan(u: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, A_log
     if N.use_native(u):
         y = torch.empty((T, H * P), dtype=torch.float32, device=u.device)
         N.mcall("mx_ssm_scan", N.ptr(u), C, N.ptr(_rows(dt_raw)), dt_raw.stride(0), _dt(dt_raw), N.ptr(dt_bias),
-                N.ptr(A_log), N.ptr(D), N.ptr(state), N.ptr(cu), N.ptr(slot), N.ptr(pos), N.ptr(y), S, H, P, Ns, G,
+                N.ptr(A_log), N.ptr(D), N.ptr(state), N.ptr(cu), N.ptr(slot), N.ptr(pos), N.ptr(y), S, H, P, Ns, G, T,
                 N.stream())
         return y
     y = torch.zeros((T, H * P), dtype=torch.float32)

@@ -122,23 +122,24 @@ def test_no_feed_forward_no_mask_single_groups(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-def test_other_sizes(device):
-    """Sizes unlike the small default: odd head counts, state and value sizes that fill no wave, a
-    window longer than a page, partial rotation, five-tap convolution, many experts."""
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_other_sizes(device, dtype):
+    """Sizes unlike the small default: odd head counts, state and value sizes that fill no wave, an odd
+    latent width, a window longer than a page, five-tap convolution, many experts."""
     cfgd = small_config("aMmA", width=80, vocab=97, heads=5)
     for l in cfgd["layers"]:
         if l["type"] == "latent_attention":
-            l["mixer"].update(dim=12, rot_dim=6, vdim=28, kv_rank=34, q_rank=44, mask={"size": 70}, scale=0.31,
+            l["mixer"].update(dim=12, rot_dim=6, vdim=28, kv_rank=35, q_rank=44, mask={"size": 70}, scale=0.31,
                               rot={"base": 500.0, "dims": 6})
         else:
             l["mixer"].update(heads=3, vdim=33, state=50, groups=3, norm_groups=3, conv=5)
         if l["mlp"]["kind"] == "moe":
             l["mlp"]["router"].update(experts=70, identity=3, top=5)
             l["mlp"]["expert"].update(ff=20, limit=0.7)
-    eng, sd = build(cfgd, device, torch.float32, blocks_=8)
+    eng, sd = build(cfgd, device, dtype, blocks_=8)
     poison(eng)
     toks = tokens(150, cfgd["vocab"], 7)
-    close(run_whole(eng, "r", toks), oracle.forward(cfgd, sd, toks, torch.float64), torch.float32)
+    close(run_whole(eng, "r", toks), oracle.forward(cfgd, sd, toks, torch.float64), dtype)
 
 
 # ---------------------------------------------------------------------------------------------------
