@@ -261,9 +261,13 @@ latent_attend_mfma_kernel(const bf16* __restrict__ q_lat, const bf16* __restrict
   for (int nt = 0; nt < NTM; ++nt) o[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  // zero the padding columns / rows once: staging below only writes real elements of staged rows
-  for (int e = threadIdx.x; e < MKT * ldk; e += 256) kt_lds[e] = (bf16)0.f;
-  for (int e = threadIdx.x; e < NT * 16 * MLDV; e += 256) vt_lds[e] = (bf16)0.f;
+  // zero the padding columns / rows once (staging only writes real elements); nothing to do when the
+  // 16-byte staging path covers every column the MFMAs read
+  if ((D & 31) != 0 || (R & 15) != 0) {
+    unsigned* z = reinterpret_cast<unsigned*>(smem);
+    const int words = (MKT * ldk + NT * 16 * MLDV) / 2;
+    for (int e = threadIdx.x; e < words; e += 256) z[e] = 0u;
+  }
 
   int k_begin = (lo / MKT) * MKT, k_end = p_last;     // first tile start, last key
   if (nsplit > 1) {
