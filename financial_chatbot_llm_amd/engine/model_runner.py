@@ -482,8 +482,10 @@ class ModelRunner:
         """Does sampling the rows ``h`` run inside the LM head (fused K11 + K12)?  TP=1 only: under TP
         the vocabulary is sharded and the logits are all-gathered before sampling."""
         m = self.model
+        # (layered decoders come in arbitrary widths: they take the fused kernels only at the widths those
+        # were measured at, multiples of 256, and logits + sampler otherwise)
         return (getattr(m, "tp_size", 1) == 1 and hasattr(m, "lm_weight") and h.dtype == torch.bfloat16
-                and ops.fused_lm_head_ok(h, m.lm_weight()))
+                and (not self.seg or h.shape[1] % 256 == 0) and ops.fused_lm_head_ok(h, m.lm_weight()))
 
     def _lm_tiled(self):
         f = getattr(self.model, "lm_tiled", None)

@@ -280,6 +280,13 @@ def test_far_key_in_a_long_prompt_chunk(device):
         out = mx.latent_attend(q.to(device), torch.zeros(len(pos), H, Dr, device=device), cache.to(device), cu.to(device),
                                pos.to(device), perm.to(device), window, 1.0, len(pos)).cpu()
         assert bool((out[:, :, 1] > 25.0).all()) == hit
+        # the same far key seen from single decoded rows (bf16: the split-key form on the GPU)
+        for dt in DTYPES:
+            one = mx.latent_attend(q[:1].to(dt).to(device), torch.zeros(1, H, Dr, dtype=dt, device=device),
+                                   cache.to(dt).to(device), torch.tensor([0, 1], dtype=torch.int32, device=device),
+                                   torch.tensor([399], dtype=torch.int32, device=device), perm.to(device), window, 1.0,
+                                   1).float().cpu()
+            assert bool((one[:, :, 1] > 25.0).all()) == hit
 
 
 @pytest.mark.gpu
