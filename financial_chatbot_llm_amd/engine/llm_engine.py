@@ -56,6 +56,11 @@ def plan_kv_blocks(cfg: EngineConfig, model, device) -> int:
     free, _ = torch.cuda.mem_get_info(device)
     reserve = 6 << 30  # activations, hipBLASLt workspaces, graph pools
     n = int(max(free - reserve, 0) * cfg.kv_mem_fraction) // per_block
+    if hasattr(model, "kv_bytes_per_block"):
+        # layered decoders: pages can be very small (or, without attention layers, empty), and nothing
+        # outlives its sequence when prefix caching is off -- the live maximum is all that is useful
+        pages_live = cfg.max_num_seqs * ((cfg.max_model_len + KV_BS - 1) // KV_BS)
+        n = min(n, pages_live if getattr(model, "has_state", False) else 4 * pages_live)
     return max(n, 16)
 
 
