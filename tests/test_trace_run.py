@@ -1,0 +1,54 @@
+"""bin/trace_run end to end on the CPU: a model directory written here (config.json + model.safetensors of
+a small random Gezavik model), a few steps on standard input, logits files against the plain oracle."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import gezavik_oracle as oracle
+from financial_chatbot_llm_amd.models.configs import layered_config
+from financial_chatbot_llm_amd.models.gezavik import GezavikModel
+from test_gezavik import random_weights, small_config, tokens
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_cli(tmp_path, dtype):
+    from safetensors.torch import save_file
+    cfgd = small_config("AmaM", width=64, vocab=120, heads=2)
+    model_dir, out_dir = tmp_path / "model", tmp_path / "out"
+    model_dir.mkdir()
+    (model_dir / "config.json").write_text(json.dumps(cfgd))
+    sd = random_weights(GezavikModel(layered_config(cfgd, "t"), device="cpu"), 3)
+    save_file({k: v.contiguous() for k, v in sd.items()}, str(model_dir / "model.safetensors"))
+    a, b = tokens(75, 120, 1), tokens(9, 120, 2)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:66], "want": [0, 65]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[:2], "want": []}, {"id": "a", "tokens": a[66:67], "want": [0]}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[67:], "want": [7]}, {"id": "b", "tokens": b[2:], "want": [6]}],
+         "end": ["a", "b"]},
+    ]
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", str(model_dir), "--dtype", dtype,
+                        "--out", str(out_dir), "--max-tokens", "192", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert not (out_dir / "1.f32").exists() or np.fromfile(out_dir / "1.f32", "<f4").size == 120
+    wa = oracle.forward(cfgd, sd, a, torch.float64)
+    wb = oracle.forward(cfgd, sd, b, torch.float64)
+    tol = 3e-4 if dtype == "float32" else 6e-2
+
+    def ok(got, want):
+        want = want.float().numpy()
+        assert np.abs(got - want).max() / np.abs(want).max() < tol
+
+    g0 = np.fromfile(out_dir / "0.f32", "<f4").reshape(2, 120)
+    ok(g0[0], wa[0]); ok(g0[1], wa[65])
+    ok(np.fromfile(out_dir / "1.f32", "<f4").reshape(1, 120)[0], wa[66])
+    g2 = np.fromfile(out_dir / "2.f32", "<f4").reshape(2, 120)
+    ok(g2[0], wa[74]); ok(g2[1], wb[8])
