@@ -8,6 +8,8 @@ from .activation import gelu_, silu_mul
 from .attention import (KV_BS, DecodeWorkspace, decode, default_scale, prefill, rope_cos_sin, rope_kv_write,
                         write_kv_ref)
 from .embedding import embedding
+from .mixers import (conv_silu, embed_f32, glu_clamp, group_norm, latent_attend, latent_prep, moe_combine, relu2,
+                     residual_norm, route_biased, ssm_scan)
 from .norm import layer_norm, rms_norm
 from .retrieval import filtered_topk
 from .sampling import (apply_top_k_top_p, fused_lm_head_ok, lm_head_sample, lm_head_sample_shard, lm_head_stream_sample,
@@ -16,4 +18,5 @@ from .sampling import (apply_top_k_top_p, fused_lm_head_ok, lm_head_sample, lm_h
 
 __all__ = ["gelu_", "silu_mul", "KV_BS", "DecodeWorkspace", "decode", "default_scale", "prefill", "rope_cos_sin",
            "rope_kv_write", "write_kv_ref", "embedding", "layer_norm", "rms_norm", "filtered_topk",
-           "apply_top_k_top_p", "sample"]
+           "apply_top_k_top_p", "sample", "conv_silu", "embed_f32", "glu_clamp", "group_norm", "latent_attend",
+           "latent_prep", "moe_combine", "relu2", "residual_norm", "route_biased", "ssm_scan"]

@@ -31,3 +31,7 @@ def gelu_(x: torch.Tensor) -> torch.Tensor:
         return x
     x.copy_(torch.nn.functional.gelu(x.float()).to(x.dtype))
     return x
+
+
+# relu^2 and the clamped gated unit g * sigmoid(alpha g) * (u + 1) (layered decoders; csrc/mixers)
+from .mixers import glu_clamp, relu2  # noqa: E402,F401

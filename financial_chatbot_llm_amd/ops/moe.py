@@ -447,3 +447,8 @@ def moe_decode_fp8(h: torch.Tensor, router_logits: torch.Tensor, w13t: torch.Ten
     out = torch.empty_like(h)
     N.call("penny_moe_combine", N.ptr(ws.y2), N.ptr(ws.inv), T, top_k, H, N.ptr(out), st)
     return out
+
+
+# Biased top-k routing (choice by score + correction, weights = plain scores, identity experts) and
+# its weighted combine: used by the layered decoders' routed feed-forward; kernels in csrc/mixers.
+from .mixers import moe_combine, route_biased  # noqa: E402,F401

@@ -60,3 +60,8 @@ def layer_norm(x: torch.Tensor, g: torch.Tensor, b: torch.Tensor, eps: float,
         return out
     xf = x.float() + (residual.float() if residual is not None else 0.0)
     return torch.nn.functional.layer_norm(xf, (H,), g.float(), b.float(), eps).to(x.dtype)
+
+
+# f32 residual stream: parallel-block update fused with the next RMS norm, and RMS norms over strided
+# slices / equal groups / with a SiLU gate first (layered decoders; kernels in csrc/mixers)
+from .mixers import group_norm, residual_norm  # noqa: E402,F401
