@@ -23,7 +23,8 @@ constexpr int MAX_TAPS = 8;
 // grid (ceil(C/256), ceil(max_len/CONV_TT), S)
 template <typename T>
 __global__ void conv_silu_kernel(const T* __restrict__ in, long si, const float* __restrict__ w,
-                                 const float* __restrict__ bias, const float* __restrict__ state,
+                                 const float* __restrict__ bias, const float* __restrict__ in_bias, int act,
+                                 const float* __restrict__ state,
                                  const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ pos,
                                  float* __restrict__ out, int C, int K) {
   const int s = blockIdx.z;
@@ -37,6 +38,7 @@ __global__ void conv_silu_kernel(const T* __restrict__ in, long si, const float*
   const bool fresh = pos[r0] == 0;
   const float* st = state + (long)sl * (K - 1) * C;
   float wk[MAX_TAPS], win[MAX_TAPS];
+  const float ib = in_bias != nullptr ? in_bias[c] : 0.f;   // added to every real input (the history holds biased inputs)
 #pragma unroll
   for (int k = 0; k < MAX_TAPS; ++k) {
     wk[k] = k < K ? w[(long)c * K + k] : 0.f;
@@ -47,7 +49,7 @@ __global__ void conv_silu_kernel(const T* __restrict__ in, long si, const float*
   for (int k = 0; k < MAX_TAPS - 1; ++k) {
     if (k < K - 1) {
       const int j = t0 - (K - 1) + k;          // local index, may be < 0
-      win[k + 1] = j >= 0 ? ldf(in + (long)(r0 + j) * si + c) : (fresh ? 0.f : st[(long)(K - 1 + j) * C + c]);
+      win[k + 1] = j >= 0 ? ldf(in + (long)(r0 + j) * si + c) + ib : (fresh ? 0.f : st[(long)(K - 1 + j) * C + c]);
     }
   }
   const float b = bias != nullptr ? bias[c] : 0.f;
@@ -56,13 +58,13 @@ __global__ void conv_silu_kernel(const T* __restrict__ in, long si, const float*
 #pragma unroll
     for (int k = 0; k < MAX_TAPS - 1; ++k) win[k] = win[k + 1];
     // after the shift the newest input goes to tap K-1
-    const float v = ldf(in + (long)(r0 + i) * si + c);
+    const float v = ldf(in + (long)(r0 + i) * si + c) + ib;
 #pragma unroll
     for (int k = 0; k < MAX_TAPS; ++k) if (k == K - 1) win[k] = v;
     float acc = b;
 #pragma unroll
     for (int k = 0; k < MAX_TAPS; ++k) if (k < K) acc += wk[k] * win[k];
-    out[(long)(r0 + i) * C + c] = mx_silu(acc);
+    out[(long)(r0 + i) * C + c] = act == 1 ? mx_silu(acc) : acc;
   }
 }
 
@@ -70,7 +72,7 @@ __global__ void conv_silu_kernel(const T* __restrict__ in, long si, const float*
 // of the same step (same stream).  One thread owns a channel's K-1 entries and walks them upward,
 // reading entry j + n before it writes entry j, so the shift is safe in place.
 template <typename T>
-__global__ void conv_state_kernel(const T* __restrict__ in, long si, float* __restrict__ state,
+__global__ void conv_state_kernel(const T* __restrict__ in, long si, const float* __restrict__ in_bias, float* __restrict__ state,
                                   const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ pos,
                                   int C, int K) {
   const int s = blockIdx.y;
@@ -85,7 +87,7 @@ __global__ void conv_state_kernel(const T* __restrict__ in, long si, float* __re
   for (int j = 0; j < K - 1; ++j) {
     const int i = n - (K - 1) + j;             // local index of the input that lands in entry j
     float v;
-    if (i >= 0) v = ldf(in + (long)(r0 + i) * si + c);
+    if (i >= 0) v = ldf(in + (long)(r0 + i) * si + c) + (in_bias != nullptr ? in_bias[c] : 0.f);
     else v = fresh ? 0.f : st[(long)(j + n) * C + c];
     st[(long)j * C + c] = v;
   }
@@ -323,19 +325,26 @@ ssm_scan_kernel(const float* __restrict__ u, int C, const TD* __restrict__ dt_ra
 }  // namespace
 
 // in: [rows, C] slice (row stride si) of the in-projection; out: f32 [rows, C]; state f32 [slots, K-1, C]
+// act: 0 none, 1 SiLU; in_bias (optional, [C]) is added to every input before the convolution
+MX_API int mx_conv_act(const void* in, long si, int dt, const float* w, const float* bias, const float* in_bias, int act,
+                       float* state, const int* cu, const int* slot, const int* pos, float* out, int S, int max_len,
+                       int C, int K, hipStream_t st) {
+  if (S <= 0 || max_len <= 0) return 0;
+  if (K < 1 || K > MAX_TAPS || act < 0 || act > 1) return (int)hipErrorInvalidValue;
+  dim3 grid((C + 255) / 256, (max_len + CONV_TT - 1) / CONV_TT, S);
+  MX_DISPATCH(dt, TT, conv_silu_kernel<TT><<<grid, 256, 0, st>>>((const TT*)in, si, w, bias, in_bias, act, state, cu,
+                                                                 slot, pos, out, C, K));
+  if (K > 1) {
+    dim3 g2((C + 255) / 256, S);
+    MX_DISPATCH(dt, TT, conv_state_kernel<TT><<<g2, 256, 0, st>>>((const TT*)in, si, in_bias, state, cu, slot, pos, C, K));
+  }
+  MX_RETURN_LAUNCH();
+}
+
 MX_API int mx_conv_silu(const void* in, long si, int dt, const float* w, const float* bias, float* state,
                         const int* cu, const int* slot, const int* pos, float* out, int S, int max_len, int C, int K,
                         hipStream_t st) {
-  if (S <= 0 || max_len <= 0) return 0;
-  if (K < 1 || K > MAX_TAPS) return (int)hipErrorInvalidValue;
-  dim3 grid((C + 255) / 256, (max_len + CONV_TT - 1) / CONV_TT, S);
-  MX_DISPATCH(dt, TT, conv_silu_kernel<TT><<<grid, 256, 0, st>>>((const TT*)in, si, w, bias, state, cu, slot, pos,
-                                                                 out, C, K));
-  if (K > 1) {
-    dim3 g2((C + 255) / 256, S);
-    MX_DISPATCH(dt, TT, conv_state_kernel<TT><<<g2, 256, 0, st>>>((const TT*)in, si, state, cu, slot, pos, C, K));
-  }
-  MX_RETURN_LAUNCH();
+  return mx_conv_act(in, si, dt, w, bias, nullptr, 1, state, cu, slot, pos, out, S, max_len, C, K, st);
 }
 
 // u f32 [rows, C = H*P + 2*G*N]; dt_raw [rows, H] slice (stride sdt, type dt_code); state f32

@@ -1,7 +1,7 @@
-"""Model families: Llama-3 (8B/70B), Mixtral-8x7B MoE, BERT/bge encoder."""
+"""Model families: Llama-3 (8B/70B), Mixtral-8x7B MoE, BERT/bge encoder, and the layered decoders Gezavik and Sigudra."""
 from __future__ import annotations
 
-from .configs import REGISTRY, ModelConfig, get_model_config
+from .configs import LAYERED_ARCHS, REGISTRY, ModelConfig, get_model_config
 
 
 def build_model(engine_cfg, device, seed: int = 0):
@@ -10,7 +10,7 @@ def build_model(engine_cfg, device, seed: int = 0):
     from .llama import LlamaModel
     from .mixtral import MixtralModel
     cfg = get_model_config(engine_cfg.model)
-    if cfg.arch == "gezavik":
+    if cfg.arch in LAYERED_ARCHS:
         return _build_layered(cfg, engine_cfg, device, seed)
     if cfg.arch == "mixtral":
         model = MixtralModel(cfg, device=device, fp8=getattr(engine_cfg, "dtype", "bf16") == "fp8",
@@ -41,7 +41,9 @@ def _build_layered(cfg, engine_cfg, device, seed: int):
     import torch
 
     from .gezavik import GezavikModel
+    from .sigudra import SigudraModel
     from .weights import read_safetensors
+    cls = {"gezavik": GezavikModel, "sigudra": SigudraModel}[cfg.arch]
     if getattr(engine_cfg, "tp_size", 1) > 1:
         raise ValueError(f"{cfg.name}: tensor parallelism is not implemented for layered decoders")
     dtype = str(getattr(engine_cfg, "dtype", "bf16")).lower()
@@ -51,7 +53,7 @@ def _build_layered(cfg, engine_cfg, device, seed: int):
     if f32:      # no reduced-precision matrix mode for f32 products
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
-    model = GezavikModel(cfg, device=device, dtype=torch.float32 if f32 else torch.bfloat16)
+    model = cls(cfg, device=device, dtype=torch.float32 if f32 else torch.bfloat16)
     src = engine_cfg.weights or (engine_cfg.model if os.path.isdir(engine_cfg.model) else None)
     if src:
         model.load_state(read_safetensors(src))

@@ -62,36 +62,69 @@ class KVCache:
 
 
 class HybridCache:
-    """Per-layer memory of a layered decoder: a paged latent cache for every attention layer and a
-    state slot array for every recurrent layer, behind the engine's one page table and one slot id
-    per sequence.
+    """Per-layer memory of a layered decoder: paged row caches for attention layers and state slot
+    arrays for recurrent layers, behind the engine's one page table and one slot id per sequence.
 
-    ``layers[i]`` is ``("latent", rows)`` with rows [num_blocks * 64, row_width] in the activation
-    dtype, or ``("state", conv, ssm)`` with f32 conv [slots, taps - 1, channels] and f32 ssm
-    [slots, heads, vdim, state].  Pages and slots are handed on uncleared: a latent row is written
-    before any query may see it, and a sequence's first segment starts from zero state."""
+    A layer's spec -> its entry in ``layers``:
 
-    def __init__(self, specs, num_blocks: int, num_slots: int, dtype, device):
+    * ``("latent", w)`` / ``("rows", w)`` -> ``(kind, rows)``, rows [num_blocks * 64, w] in the
+      activation dtype (one cache row per token: a key/value latent, or [keys | values]);
+    * ``("state", taps, channels, heads, vdim, state)`` -> ``("state", conv, ssm)``, f32 conv
+      [slots, taps - 1, channels] and ssm [slots, heads, vdim, state];
+    * ``("slots", {name: shape})`` -> ``("slots", {name: f32 [slots, *shape]})``;
+    * ``("pair", spec_a, spec_b)`` -> ``("pair", entry_a, entry_b)`` (two mixers side by side).
+
+    ``slot_arrays`` ({name: (dtype, shape)}) are per-slot records of the model as a whole
+    (``model[name]``: [slots, *shape]), e.g. the last token of each sequence.  Pages and slots are
+    handed on uncleared: a cache row is written before any query may see it, and a sequence's
+    first segment starts from zero state."""
+
+    def __init__(self, specs, num_blocks: int, num_slots: int, dtype, device, slot_arrays=None):
         self.num_blocks, self.num_slots = num_blocks, num_slots
-        self.layers = []
+        self.dtype, self.device = dtype, device
+        self.layers = [self._make(sp) for sp in specs]
+        self.model = {n: torch.zeros((num_slots, *shape), dtype=dt, device=device)
+                      for n, (dt, shape) in (slot_arrays or {}).items()}
+
+    def _make(self, sp):
+        nb, ns, dev = self.num_blocks, self.num_slots, self.device
+        if sp[0] in ("latent", "rows"):
+            return (sp[0], torch.zeros((nb * KV_BS, sp[1]), dtype=self.dtype, device=dev))
+        if sp[0] == "state":
+            _, taps, channels, heads, vdim, nstate = sp
+            return ("state", torch.zeros((ns, max(taps - 1, 1), channels), dtype=torch.float32, device=dev),
+                    torch.zeros((ns, heads, vdim, nstate), dtype=torch.float32, device=dev))
+        if sp[0] == "slots":
+            return ("slots", {n: torch.zeros((ns, *shape), dtype=torch.float32, device=dev) for n, shape in sp[1].items()})
+        if sp[0] == "pair":
+            return ("pair", self._make(sp[1]), self._make(sp[2]))
+        return (sp[0],)
+
+    @staticmethod
+    def _flat(specs):
         for sp in specs:
-            if sp[0] == "latent":
-                self.layers.append(("latent", torch.zeros((num_blocks * KV_BS, sp[1]), dtype=dtype, device=device)))
-            elif sp[0] == "state":
-                _, taps, channels, heads, vdim, nstate = sp
-                self.layers.append(("state",
-                                    torch.zeros((num_slots, max(taps - 1, 1), channels), dtype=torch.float32, device=device),
-                                    torch.zeros((num_slots, heads, vdim, nstate), dtype=torch.float32, device=device)))
+            if sp[0] == "pair":
+                yield from HybridCache._flat(sp[1:])
             else:
-                self.layers.append((sp[0],))
+                yield sp
 
     @staticmethod
     def bytes_per_block(specs, elt: int) -> int:
-        return max(1, sum(KV_BS * sp[1] * elt for sp in specs if sp[0] == "latent"))
+        return max(1, sum(KV_BS * sp[1] * elt for sp in HybridCache._flat(specs) if sp[0] in ("latent", "rows")))
 
     @staticmethod
     def bytes_per_slot(specs) -> int:
-        return sum(4 * (max(sp[1] - 1, 1) * sp[2] + sp[3] * sp[4] * sp[5]) for sp in specs if sp[0] == "state")
+        n = 0
+        for sp in HybridCache._flat(specs):
+            if sp[0] == "state":
+                n += 4 * (max(sp[1] - 1, 1) * sp[2] + sp[3] * sp[4] * sp[5])
+            elif sp[0] == "slots":
+                for shape in sp[1].values():
+                    k = 4
+                    for d in shape:
+                        k *= d
+                    n += k
+        return n
 
 
 def param_seed(base: int, name: str) -> int:

@@ -6,9 +6,25 @@ normed input ``h`` and return a sublayer output, with their sizes and constants 
 * :class:`LatentAttentionMixer` -- attention whose keys and values are up-projections of one cached
   latent per token plus one shared rotated key part; runs in the latent space over a paged latent
   cache with a sliding window and a per-head sigmoid output gate.
-* :class:`DenseFF` -- up, activation, down.
+* :class:`ChannelDeltaMixer` -- gated delta rule with one decay per head and key channel (short
+  convolutions on q, k, v; unit-norm q and k; low-rank decay and output-gate projections).
+* :class:`GLAMixer` -- gated linear attention: the same matrix state with a plain k v^T write and a
+  decay sigmoid(.)^(1/tau) per key channel.
+* :class:`WindowAttentionMixer` -- softmax attention over a paged [keys | values] row cache with
+  grouped key/value heads, RMS norm over the whole query / key projection, a sliding window, no
+  positional rotation and a per-head sigmoid output gate.
+* :class:`GatedLRUMixer` -- real-gated linear recurrent unit block (GeLU branch times a
+  convolved, block-diagonally gated diagonal recurrence).
+* :class:`ParallelMixer` -- two of the above side by side on the same input; the layer combines their
+  RMS-normed outputs.
+* :class:`DenseFF` -- up, activation, down; optionally gated (act(gate) * up).
 * :class:`RoutedFF` -- mixture of clamped gated experts with biased top-k choice, identity experts
   and an always-on shared expert.
+* :class:`InputScaledRoutedFF` -- mixture of gated experts chosen by independent sigmoid scores, the
+  score multiplying the expert's input.
+
+A shape entry of ``None`` in ``shapes()`` is a size only the checkpoint's tensor gives (a low-rank
+projection's rank).
 
 Every block declares the rows it needs from a fused in-projection (``in_weight``): a layer stacks
 its mixer's and its feed-forward's rows into ONE GEMM over ``h`` and hands each block its column
@@ -145,25 +161,33 @@ class LatentAttentionMixer:
 
 
 class DenseFF:
-    """W_down act(W_up h); ``act``: "relu2" (the square of relu)."""
+    """W_down act(W_up h), ``act`` = "relu2" (the square of relu); or, ``gated``,
+    W_down (act(W_gate h) * (W_up h)) with ``act`` in silu | gelu_tanh."""
 
-    def __init__(self, spec: Dict, width: int, act: str = "relu2"):
-        self.ff, self.width, self.act = int(spec["ff"]), width, act
-        self.in_rows = self.ff
-        if act != "relu2":
-            raise ValueError(f"unknown activation {act!r}")
+    def __init__(self, spec: Dict, width: int, act: str = "relu2", gated: bool = False):
+        self.ff, self.width, self.act, self.gated = int(spec["ff"]), width, act, gated
+        self.in_rows = self.ff * (2 if gated else 1)
+        if (act != "relu2") != gated or act not in ("relu2", "silu", "gelu_tanh"):
+            raise ValueError(f"unknown activation {act!r} for a {'gated' if gated else 'plain'} feed-forward")
 
     def shapes(self) -> Dict[str, tuple]:
-        return {"up": (self.ff, self.width), "down": (self.width, self.ff)}
+        s = {"up": (self.ff, self.width), "down": (self.width, self.ff)}
+        if self.gated:
+            s["gate"] = (self.ff, self.width)
+        return s
 
     def load(self, get: Getter, dtype) -> torch.Tensor:
         self.down = get("down").to(dtype).contiguous()
+        if self.gated:
+            return torch.cat([get("gate"), get("up")], 0).to(dtype)
         return get("up").to(dtype)
 
     def num_bytes(self) -> int:
         return self.down.numel() * self.down.element_size()
 
     def forward(self, h: torch.Tensor, proj: torch.Tensor) -> torch.Tensor:
+        if self.gated:
+            return F.linear(mx.glu_act(proj[:, :self.ff], proj[:, self.ff:2 * self.ff], self.act), self.down)
         return F.linear(mx.relu2(proj), self.down)
 
 
@@ -240,4 +264,306 @@ class RoutedFF:
         return mx.moe_combine(ys, pos.view(T, top).to(torch.int32), idx, wts, h, shared, E)
 
 
-MIXERS = {"mamba2": Mamba2Mixer, "latent_attention": LatentAttentionMixer}
+class InputScaledRoutedFF:
+    """Mixture of ``experts`` gated feed-forwards without biases, ``top`` per token.
+
+    Router logits z = W_r h in f32, scores s = sigmoid(z) (``score``; each expert on its own); the
+    ``top`` largest are chosen and their scores are the weights, not renormalised.  The weight
+    multiplies the expert's INPUT: out = sum_e expert_e(s_e h), expert(x) = W_d (act(W_g x) * (W_u x)).
+    Since W (s h) = s (W h), the experts' first projections run on h itself and the activation
+    kernel applies s to both halves."""
+
+    def __init__(self, spec: Dict, width: int, act: str = "silu", score: str = "sigmoid"):
+        r = spec["router"]
+        self.E, self.top = int(r["experts"]), int(r["top"])
+        self.F = int(spec["expert"]["ff"])
+        self.act, self.score, self.width = act, score, width
+        self.in_rows = 0
+        if not 1 <= self.top <= self.E:
+            raise ValueError("routed feed-forward: 1 <= top <= experts")
+
+    def shapes(self) -> Dict[str, tuple]:
+        s = {"router": (self.E, self.width)}
+        for e in range(self.E):
+            s.update({f"e{e}.gate": (self.F, self.width), f"e{e}.up": (self.F, self.width),
+                      f"e{e}.down": (self.width, self.F)})
+        return s
+
+    def load(self, get: Getter, dtype) -> Optional[torch.Tensor]:
+        self.router = get("router").float().contiguous()
+        self.w13 = torch.stack([torch.cat([get(f"e{e}.gate"), get(f"e{e}.up")], 0) for e in range(self.E)]).to(dtype)
+        self.w2 = torch.stack([get(f"e{e}.down") for e in range(self.E)]).to(dtype).contiguous()
+        return None
+
+    def num_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.router, self.w13, self.w2))
+
+    def forward(self, h: torch.Tensor, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
+        T, W = h.shape
+        E, top, Fe = self.E, self.top, self.F
+        wts, idx = mx.route_scores(F.linear(h.float(), self.router), top, self.score)
+        ones = torch.ones_like(wts)
+        if T * top <= DENSE_MAX_PAIRS or _capturing(h):
+            # every expert over every row; rows an expert was not chosen for get scale 0 and are not read
+            rows = torch.arange(T, device=h.device)[:, None]
+            pos = idx.long() * T + rows
+            scale = torch.zeros(E * T, dtype=torch.float32, device=h.device).scatter_(0, pos.reshape(-1), wts.reshape(-1))
+            gu = torch.bmm(h.unsqueeze(0).expand(E, T, W), self.w13.transpose(1, 2)).view(E * T, 2 * Fe)
+            act = mx.glu_act(gu[:, :Fe], gu[:, Fe:], self.act, scale)
+            ys = torch.bmm(act.view(E, T, Fe), self.w2.transpose(1, 2)).view(E * T, W)
+            return mx.moe_combine(ys, pos.to(torch.int32), idx, ones, h, None, E)
+        flat = idx.reshape(-1).long()
+        order = torch.argsort(flat, stable=True)
+        offs = [0] + torch.bincount(flat, minlength=E).cumsum(0).tolist()              # host read of the buckets
+        xs = h.index_select(0, order // top)
+        sc = wts.reshape(-1)[order].contiguous()
+        ys = torch.empty((T * top, W), dtype=h.dtype, device=h.device)
+        for e in range(E):
+            a, b = offs[e], offs[e + 1]
+            if b > a:
+                gu = F.linear(xs[a:b], self.w13[e])
+                torch.mm(mx.glu_act(gu[:, :Fe], gu[:, Fe:], self.act, sc[a:b]), self.w2[e].t(), out=ys[a:b])
+        pos = torch.empty_like(order)
+        pos[order] = torch.arange(order.numel(), device=order.device)
+        return mx.moe_combine(ys, pos.view(T, top).to(torch.int32), idx, ones, h, None, E)
+
+
+def _f32(get: Getter, name: str) -> torch.Tensor:
+    return get(name).float().contiguous()
+
+
+class ChannelDeltaMixer:
+    """Gated delta rule with a decay per head and key channel.
+
+    q = W_q h, k = W_k h ([kv_heads, dim]), v = W_v h ([heads, vdim]); each through a causal
+    per-channel convolution (no bias) and SiLU; q and k become unit vectors per head (q also times
+    dim^-1/2); b = sigmoid(W_b h) per head; g = exp(-exp(A_log_h) softplus(W_a2 W_a1 h + dt_bias)) per
+    head and key channel.  Per head, on the f32 state S [dim, vdim]:
+    S <- g S;  u = b (v - S^T k);  S <- S + k u^T;  o = S^T q.
+    Output: o / rms(o) * w_norm * sigmoid(W_g2 W_g1 h), then W_o.  Slot state: S and the last
+    taps - 1 inputs of the three convolutions."""
+    kind = "channel_delta"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.H, self.G = int(spec["heads"]), int(spec.get("kv_heads", spec["heads"]))
+        self.D, self.P, self.K = int(spec["dim"]), int(spec["vdim"]), int(spec["conv"])
+        self.ra, self.rg = spec.get("decay_rank"), spec.get("gate_rank")      # set by the checkpoint's shapes
+        self.width, self.eps = width, eps
+        if self.H % self.G or not 1 <= self.K <= 8 or self.D > 512:
+            raise ValueError("channel_delta: heads must split into kv_heads, 1 <= conv taps <= 8, dim <= 512")
+        self.nq, self.nv = self.G * self.D, self.H * self.P
+        self.C = 2 * self.nq + self.nv
+
+    def shapes(self) -> Dict[str, tuple]:
+        W = self.width
+        return {"q": (self.nq, W), "q.conv": (self.nq, self.K), "k": (self.nq, W), "k.conv": (self.nq, self.K),
+                "v": (self.nv, W), "v.conv": (self.nv, self.K), "b": (self.H, W), "A_log": (self.H,), "norm": (self.P,),
+                "a1": (self.ra, W), "a2": (self.H * self.D, self.ra), "dt_bias": (self.H * self.D,),
+                "g1": (self.rg, W), "g2": (self.nv, self.rg), "o": (W, self.nv)}
+
+    def cache_spec(self):
+        return ("slots", {"conv": (max(self.K - 1, 1), self.C), "S": (self.H, self.D, self.P)})
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.conv_w = torch.cat([_f32(get, "q.conv"), _f32(get, "k.conv"), _f32(get, "v.conv")], 0).contiguous()
+        self.A_log, self.dt_bias, self.norm_w = _f32(get, "A_log"), _f32(get, "dt_bias"), _f32(get, "norm")
+        self.a2 = _f32(get, "a2")                 # the decay's pre-activation is computed in f32
+        self.g2 = get("g2").to(dtype).contiguous()
+        self.o = get("o").to(dtype).contiguous()
+        self.ra, self.rg = self.a2.shape[1], self.g2.shape[1]
+        self.in_rows = self.C + self.H + self.ra + self.rg
+        return torch.cat([get("q"), get("k"), get("v"), get("b"), get("a1"), get("g1")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.conv_w, self.a2, self.g2, self.o))
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        st = cache[1]
+        C, H, nq = self.C, self.H, self.nq
+        u = mx.conv_act(proj[:, :C], self.conv_w, None, st["conv"], meta.seg_cu, meta.seg_state, positions,
+                        meta.seg_max_len, "silu")
+        beta = proj[:, C:C + H]
+        a = F.linear(proj[:, C + H:C + H + self.ra].float(), self.a2)
+        o = mx.matrix_scan(u[:, :nq], u[:, nq:2 * nq], u[:, 2 * nq:], a, self.dt_bias, st["S"], meta.seg_cu,
+                           meta.seg_state, positions, H, self.G, self.D, self.P, "delta", A_log=self.A_log, beta=beta)
+        gate = F.linear(proj[:, C + H + self.ra:C + H + self.ra + self.rg], self.g2)
+        return F.linear(mx.head_norm_gate(o, self.norm_w, self.eps, gate, H, "sigmoid", proj.dtype), self.o)
+
+
+class GLAMixer:
+    """Gated linear attention: q = W_q h dim^-1/2, k = W_k h ([heads, dim]), v = W_v h ([heads, vdim]);
+    decay per head and key channel alpha = sigmoid(W_a2 W_a1 h + b_a2)^(1/tau); on the f32 state
+    S [dim, vdim]: S <- diag(alpha) S + k v^T, o = S^T q.  Output: RMS norm of each head's o times
+    w_norm, times silu(W_g h), then W_o."""
+    kind = "gla"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.H, self.D, self.P = int(spec["heads"]), int(spec["dim"]), int(spec["vdim"])
+        self.tau = float(spec.get("tau", 1.0))
+        self.ra = spec.get("decay_rank")
+        self.width, self.eps = width, eps
+        if self.D > 512 or self.tau <= 0:
+            raise ValueError("gla: dim <= 512 and tau > 0")
+        self.nq, self.nv = self.H * self.D, self.H * self.P
+
+    def shapes(self) -> Dict[str, tuple]:
+        W = self.width
+        return {"q": (self.nq, W), "k": (self.nq, W), "v": (self.nv, W), "g": (self.nv, W), "o": (W, self.nv),
+                "norm": (self.P,), "a1": (self.ra, W), "a2": (self.nq, self.ra), "a2.b": (self.nq,)}
+
+    def cache_spec(self):
+        return ("slots", {"S": (self.H, self.D, self.P)})
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.a2, self.a2_b, self.norm_w = _f32(get, "a2"), _f32(get, "a2.b"), _f32(get, "norm")
+        self.o = get("o").to(dtype).contiguous()
+        self.ra = self.a2.shape[1]
+        self.in_rows = 2 * self.nq + 2 * self.nv + self.ra
+        return torch.cat([get("q"), get("k"), get("v"), get("g"), get("a1")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.a2, self.o))
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        st = cache[1]
+        nq, nv = self.nq, self.nv
+        a = F.linear(proj[:, 2 * nq + 2 * nv:2 * nq + 2 * nv + self.ra].float(), self.a2)
+        o = mx.matrix_scan(proj[:, :nq], proj[:, nq:2 * nq], proj[:, 2 * nq:2 * nq + nv], a, self.a2_b, st["S"],
+                           meta.seg_cu, meta.seg_state, positions, self.H, self.H, self.D, self.P, "gla", tau=self.tau)
+        gate = proj[:, 2 * nq + nv:2 * nq + 2 * nv]
+        return F.linear(mx.head_norm_gate(o, self.norm_w, self.eps, gate, self.H, "silu", proj.dtype), self.o)
+
+
+class WindowAttentionMixer:
+    """Softmax attention with ``kv_heads`` key/value heads (query head h reads head h // (H/G)), key
+    size ``dim`` and value size ``vdim``; RMS norm over the WHOLE query and key projections (before the
+    split into heads) with plain weights; no rotation; score = q . k * scale; sliding window
+    0 <= i - j < mask.size (no ``mask`` entry: plain causal); head h's output times
+    sigmoid(W_g h)_h; then W_o.  The cache holds one row [k | v] per token."""
+    kind = "window_attention"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.H, self.G = int(spec["heads"]), int(spec.get("kv_heads", spec["heads"]))
+        self.D, self.P = int(spec["dim"]), int(spec["vdim"])
+        mask = spec.get("mask") or {}
+        self.window = int(mask["size"]) if mask.get("size") else 1 << 30
+        self.scale = float(spec["scale"]) if "scale" in spec else self.D ** -0.5
+        self.width, self.eps = width, eps
+        if self.H % self.G or self.D > 512 or self.P > 512:
+            raise ValueError("window_attention: heads must split into kv_heads; dim, vdim <= 512")
+        self.nq, self.nk, self.nv = self.H * self.D, self.G * self.D, self.G * self.P
+        self.in_rows = self.nq + self.nk + self.nv + self.H
+
+    def shapes(self) -> Dict[str, tuple]:
+        W = self.width
+        return {"q": (self.nq, W), "k": (self.nk, W), "v": (self.nv, W), "q.norm": (self.nq,), "k.norm": (self.nk,),
+                "g": (self.H, W), "o": (W, self.H * self.P)}
+
+    def cache_spec(self):
+        return ("rows", self.nk + self.nv)
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.q_norm, self.k_norm = _f32(get, "q.norm"), _f32(get, "k.norm")
+        self.o = get("o").to(dtype).contiguous()
+        return torch.cat([get("q"), get("k"), get("v"), get("g")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return self.o.numel() * self.o.element_size()
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        rows = cache[1]
+        nq, nk, nv = self.nq, self.nk, self.nv
+        q = mx.qk_norm_write(proj[:, :nq], proj[:, nq:nq + nk], proj[:, nq + nk:nq + nk + nv], self.q_norm, self.k_norm,
+                             self.eps, meta.slots, rows)
+        gate = proj[:, nq + nk + nv:nq + nk + nv + self.H]
+        o = mx.window_attend(q, rows, meta.seg_cu, positions, meta.seg_bt, self.window, self.scale, meta.seg_max_len,
+                             self.H, self.G, self.D, self.P, gate=gate)
+        return F.linear(o, self.o)
+
+
+class GatedLRUMixer:
+    """Recurrent block around a real-gated linear recurrent unit of ``width`` channels:
+    y = gelu_tanh(W_y h + b_y);  u = conv(W_x h + b_x) (causal per channel, bias, no activation);
+    u in ``blocks`` equal parts, in part b: r = sigmoid(R_b u_b + c_b), i = sigmoid(I_b u_b + d_b);
+    a = exp(-8 r softplus(lam));  S <- a S + sqrt(1 - a^2) i u (from S = 0, no special first token);
+    output W_o (S * y).  Slot state: S (f32) and the last taps - 1 biased convolution inputs."""
+    kind = "gated_lru"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.R, self.B, self.K = int(spec["width"]), int(spec["blocks"]), int(spec["conv"])
+        self.width, self.eps = width, eps
+        if self.R % self.B or not 1 <= self.K <= 8:
+            raise ValueError("gated_lru: width must split into blocks, 1 <= conv taps <= 8")
+        self.bs = self.R // self.B
+        self.in_rows = 2 * self.R
+
+    def shapes(self) -> Dict[str, tuple]:
+        R, B, bs, W = self.R, self.B, self.bs, self.width
+        return {"y": (R, W), "y.b": (R,), "x": (R, W), "x.b": (R,), "conv": (R, self.K), "conv.b": (R,),
+                "ra": (B, bs, bs), "ra.b": (B, bs), "ri": (B, bs, bs), "ri.b": (B, bs), "lam": (R,), "o": (W, R)}
+
+    def cache_spec(self):
+        return ("slots", {"conv": (max(self.K - 1, 1), self.R), "S": (self.R,)})
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.y_b, self.x_b = _f32(get, "y.b"), _f32(get, "x.b")
+        self.conv_w, self.conv_b, self.lam = _f32(get, "conv"), _f32(get, "conv.b"), _f32(get, "lam")
+        # both gates' block matrices as one batched operand [B, in, 2 * out], f32 (they enter the recurrence)
+        self.w_ri = torch.cat([_f32(get, "ra").transpose(1, 2), _f32(get, "ri").transpose(1, 2)], 2).contiguous()
+        self.r_b, self.i_b = _f32(get, "ra.b").reshape(-1), _f32(get, "ri.b").reshape(-1)
+        self.o = get("o").to(dtype).contiguous()
+        return torch.cat([get("y"), get("x")], 0).to(dtype)
+
+    def num_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.conv_w, self.w_ri, self.o))
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache) -> torch.Tensor:
+        st = cache[1]
+        T, R, B, bs = proj.shape[0], self.R, self.B, self.bs
+        u = mx.conv_act(proj[:, R:2 * R], self.conv_w, self.conv_b, st["conv"], meta.seg_cu, meta.seg_state, positions,
+                        meta.seg_max_len, "none", in_bias=self.x_b)
+        z = torch.bmm(u.view(T, B, bs).transpose(0, 1), self.w_ri)             # [B, T, 2 bs]: r | i pre-activations
+        s = mx.lru_scan(u, z, B, self.r_b, self.i_b, self.lam, proj[:, :R], self.y_b, st["S"], meta.seg_cu,
+                        meta.seg_state, positions, proj.dtype)
+        return F.linear(s, self.o)
+
+
+class ParallelMixer:
+    """Two mixers side by side reading the same input (``left``: windowed attention, ``right``: gated
+    LRU block).  ``forward`` returns both outputs; the layer takes half the sum of their RMS norms
+    over the model width, with the plain weights ``left.out`` / ``right.out``."""
+    kind = "parallel"
+
+    def __init__(self, spec: Dict, width: int, eps: float):
+        self.left = WindowAttentionMixer(spec["left"], width, eps)
+        self.right = GatedLRUMixer(spec["right"], width, eps)
+        self.width = width
+        self.in_rows = self.left.in_rows + self.right.in_rows
+
+    def shapes(self) -> Dict[str, tuple]:
+        s = {f"left.{k}": v for k, v in self.left.shapes().items()}
+        s.update({f"right.{k}": v for k, v in self.right.shapes().items()})
+        s.update({"left.out": (self.width,), "right.out": (self.width,)})
+        return s
+
+    def cache_spec(self):
+        return ("pair", self.left.cache_spec(), self.right.cache_spec())
+
+    def load(self, get: Getter, dtype) -> torch.Tensor:
+        self.out_w = (_f32(get, "left.out"), _f32(get, "right.out"))
+        wl = self.left.load(lambda k: get("left." + k), dtype)
+        wr = self.right.load(lambda k: get("right." + k), dtype)
+        return torch.cat([wl, wr], 0)
+
+    def num_bytes(self) -> int:
+        return self.left.num_bytes() + self.right.num_bytes()
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, meta: AttentionMetadata, cache):
+        n = self.left.in_rows
+        return (self.left.forward(proj[:, :n], positions, meta, cache[1]),
+                self.right.forward(proj[:, n:], positions, meta, cache[2]))
+
+
+MIXERS = {"mamba2": Mamba2Mixer, "latent_attention": LatentAttentionMixer, "channel_delta": ChannelDeltaMixer,
+          "gla": GLAMixer, "window_attention": WindowAttentionMixer, "gated_lru": GatedLRUMixer,
+          "parallel": ParallelMixer}

@@ -93,6 +93,18 @@ _MIXER_SIGS = {
     "mx_route_biased": [P, P, c_int, c_int, P, P, c_int, P],
     "mx_moe_combine": [P, P, P, P, P, c_long, P, c_long, c_int, c_int, c_int, P, c_int, c_int, P],
     "mx_conv_silu": [P, c_long, c_int, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, P],
+    "mx_conv_act": [P, c_long, c_int, P, P, P, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, P],
+    "mx_embed_pairs": [P, P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, P],
+    "mx_post_norm": [P, P, c_long, P, P, c_long, P, c_int, P, c_float, P, c_int, c_int, c_int, P],
+    "mx_glu_act": [P, c_long, P, c_long, P, c_int, P, c_long, c_int, c_int, c_int, P],
+    "mx_route_scores": [P, c_int, c_int, c_int, P, P, c_int, P],
+    "mx_head_norm_gate": [P, c_long, c_int, P, c_float, P, c_long, c_int, c_int, P, c_int, c_int, c_int, c_int, P],
+    "mx_matrix_scan": [P, c_long, P, c_long, P, c_long, c_int, P, c_long, P, P, P, c_long, c_int, c_float, c_int, P, P, P,
+                       P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mx_lru_scan": [P, P, c_int, P, P, P, P, c_long, c_int, P, P, P, P, P, P, c_int, c_int, c_int, c_int, P],
+    "mx_qk_norm_write": [P, c_long, P, c_long, P, c_long, P, P, c_float, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mx_window_attend": [P, c_long, P, P, P, P, c_int, P, c_long, c_int, c_float, P, c_int, c_int, c_int, c_int, c_int,
+                         c_int, c_int, P],
     "mx_ssm_scan": [P, c_int, P, c_long, c_int, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mx_latent_prep": [P, c_long, P, c_float, P, c_int, P, P, P, P, c_long, c_int, c_int, P, c_int, c_int, c_int,
                        c_int, c_int, P],

@@ -342,3 +342,354 @@ def latent_attend(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor,
     if gate is not None:
         out = out * torch.sigmoid(gate.float())[:, :, None]
     return out.to(q_lat.dtype)
+
+
+# ----------------------------------------------------------------------------------------------
+# sequential (post-norm) blocks: hashed pair embedding, layer norm on the sublayer output
+# ----------------------------------------------------------------------------------------------
+def embed_pairs(ids: torch.Tensor, table: torch.Tensor, pair_table: Optional[torch.Tensor], mul_prev: int, mul_cur: int,
+                last_token: Optional[torch.Tensor], cu: torch.Tensor, slot: torch.Tensor, pos: torch.Tensor,
+                max_len: int) -> torch.Tensor:
+    """f32 residual stream [T, W]: ``table[id]`` plus, with a ``pair_table`` [buckets + 1, W], its row
+    ``(prev * mul_prev + id * mul_cur) mod buckets`` -- ``prev`` the token before in the same
+    sequence -- or row ``buckets`` at position 0.  ``last_token`` int32 [slots] holds every slot's
+    last token between steps (read by a segment's first row, then replaced by its last id)."""
+    T, (V, W) = ids.numel(), table.shape
+    S = cu.numel() - 1
+    ids = ids.to(torch.int32).contiguous()
+    if pair_table is None:
+        return embed_f32(ids, table)
+    B = pair_table.shape[0] - 1
+    if N.use_native(table):
+        out = torch.empty((T, W), dtype=torch.float32, device=table.device)
+        N.mcall("mx_embed_pairs", N.ptr(ids), N.ptr(table), N.ptr(pair_table), _dt(table), int(mul_prev), int(mul_cur),
+                B, N.ptr(last_token), N.ptr(cu), N.ptr(slot), N.ptr(pos), N.ptr(out), S, int(max_len), W, V, N.stream())
+        return out
+    out = table[ids.long().clamp(0, V - 1)].float()
+    cul, sll, pl, idl = cu.tolist(), slot.tolist(), pos.tolist(), ids.tolist()
+    for s in range(S):
+        a, b = cul[s], cul[s + 1]
+        if sll[s] < 0 or b <= a:
+            continue
+        for r in range(a, b):
+            if pl[r] == 0:
+                row = B
+            else:
+                prev = idl[r - 1] if r > a else int(last_token[sll[s]])
+                row = (prev * mul_prev + idl[r] * mul_cur) % B
+            out[r] += pair_table[row].float()
+        last_token[sll[s]] = idl[b - 1]
+    return out
+
+
+def _ln(v: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    mu = v.mean(-1, keepdim=True)
+    d = v - mu
+    return d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+
+
+def layer_norm_out(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """(x - mean) / sqrt(var + eps) * w of every f32 row, in ``out_dtype``."""
+    T, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    if N.use_native(x):
+        out = torch.empty((T, W), dtype=out_dtype, device=x.device)
+        N.mcall("mx_post_norm", N.ptr(x), None, 0, None, None, 0, None, 1, N.ptr(w), float(eps), N.ptr(out), _dt(out),
+                T, W, N.stream())
+        return out
+    return _ln(x, w, eps).to(out_dtype)
+
+
+def post_norm_add(x: torch.Tensor, a: torch.Tensor, w: torch.Tensor, eps: float, out_dtype: Optional[torch.dtype] = None,
+                  b: Optional[torch.Tensor] = None, wa: Optional[torch.Tensor] = None,
+                  wb: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``x`` (f32 [T, W], in place) <- x + LayerNorm(m) * w, the norm on the sublayer's output only.
+    m = a, or with a second branch m = (RMSnorm(a) * wa + RMSnorm(b) * wb) / 2 (two mixers side by
+    side).  Returns the new x rounded to ``out_dtype`` (the next sublayer's GEMM input) when one is
+    given and differs from f32, else x itself."""
+    T, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    want = out_dtype is not None and out_dtype != torch.float32
+    if N.use_native(x):
+        out = torch.empty((T, W), dtype=out_dtype, device=x.device) if want else None
+        if b is not None:
+            assert a.dtype == b.dtype
+        N.mcall("mx_post_norm", N.ptr(x), N.ptr(_rows(a)), a.stride(0), N.ptr(wa), N.ptr(_rows(b)) if b is not None else None,
+                b.stride(0) if b is not None else 0, N.ptr(wb), _dt(a), N.ptr(w), float(eps), N.ptr(out),
+                _dt(out) if want else 1, T, W, N.stream())
+        return out if want else x
+    m = a.float()
+    if b is not None:
+        rms = lambda v: v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)  # noqa: E731
+        m = 0.5 * (rms(m) * wa.float() + rms(b.float()) * wb.float())
+    x.add_(_ln(m, w, eps))
+    return x.to(out_dtype) if want else x
+
+
+ACTS = {"none": 0, "silu": 1, "gelu_tanh": 2, "sigmoid": 3}
+
+
+def _act(v: torch.Tensor, act: str) -> torch.Tensor:
+    if act == "silu":
+        return F.silu(v)
+    if act == "gelu_tanh":
+        return F.gelu(v, approximate="tanh")
+    if act == "sigmoid":
+        return torch.sigmoid(v)
+    return v
+
+
+def glu_act(gate: torch.Tensor, up: torch.Tensor, act: str, row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """act(s * gate) * (s * up) with ``s`` an optional f32 scale per row (a routed expert whose weight
+    multiplies its INPUT: the scale commutes with the two projections); ``act``: silu | gelu_tanh."""
+    T, n = gate.shape
+    if N.use_native(gate):
+        out = torch.empty((T, n), dtype=gate.dtype, device=gate.device)
+        N.mcall("mx_glu_act", N.ptr(_rows(gate)), gate.stride(0), N.ptr(_rows(up)), up.stride(0), N.ptr(row_scale),
+                ACTS[act], N.ptr(out), out.stride(0), _dt(gate), T, n, N.stream())
+        return out
+    g, u = gate.float(), up.float()
+    if row_scale is not None:
+        g, u = g * row_scale[:, None], u * row_scale[:, None]
+    return (_act(g, act) * u).to(gate.dtype)
+
+
+def route_scores(z: torch.Tensor, top: int, score: str = "sigmoid") -> Tuple[torch.Tensor, torch.Tensor]:
+    """The ``top`` largest entries of each row of the f32 router logits ``z`` (ties: the lower index)
+    and their scores -- sigmoid(z), independent per expert, or softmax(z) -- not renormalised.
+    Returns (weights f32 [T, top], indices int32 [T, top])."""
+    T, E = z.shape
+    assert z.dtype == torch.float32
+    if N.use_native(z):
+        z = z.contiguous()
+        w = torch.empty((T, top), dtype=torch.float32, device=z.device)
+        i = torch.empty((T, top), dtype=torch.int32, device=z.device)
+        N.mcall("mx_route_scores", N.ptr(z), E, top, 1 if score == "sigmoid" else 0, N.ptr(w), N.ptr(i), T, N.stream())
+        return w, i
+    s = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, -1)
+    idx = torch.topk(s, top, dim=-1).indices
+    return s.gather(1, idx), idx.to(torch.int32)
+
+
+def conv_act(inp: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, cu: torch.Tensor,
+             slot: torch.Tensor, pos: torch.Tensor, max_len: int, act: str = "silu",
+             in_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """:func:`conv_silu` with the activation as a parameter (``silu`` | ``none``) and an optional
+    bias ``in_bias`` [C] added to every input BEFORE the convolution (inputs before the sequence stay
+    zero; the slot's history holds biased inputs)."""
+    if act == "silu" and in_bias is None:
+        return conv_silu(inp, w, bias, state, cu, slot, pos, max_len)
+    T, C = inp.shape
+    K = w.shape[1]
+    S = cu.numel() - 1
+    if N.use_native(inp):
+        out = torch.empty((T, C), dtype=torch.float32, device=inp.device)
+        N.mcall("mx_conv_act", N.ptr(_rows(inp)), inp.stride(0), _dt(inp), N.ptr(w), N.ptr(bias), N.ptr(in_bias),
+                ACTS[act], N.ptr(state), N.ptr(cu), N.ptr(slot), N.ptr(pos), N.ptr(out), S, int(max_len), C, K, N.stream())
+        return out
+    out = torch.zeros((T, C), dtype=torch.float32)
+    cul, sll, pl = cu.tolist(), slot.tolist(), pos.tolist()
+    x = inp.float() + (in_bias.float() if in_bias is not None else 0.0)
+    for s in range(S):
+        a, b = cul[s], cul[s + 1]
+        if sll[s] < 0 or b <= a:
+            continue
+        hist = torch.zeros((K - 1, C)) if pl[a] == 0 else state[sll[s]].clone()
+        full = torch.cat([hist, x[a:b]])
+        acc = (full.unfold(0, K, 1) * w.float()[None]).sum(-1)
+        if bias is not None:
+            acc = acc + bias.float()
+        out[a:b] = _act(acc, act)
+        if K > 1:
+            state[sll[s]] = full[-(K - 1):]
+    return out
+
+
+# ----------------------------------------------------------------------------------------------
+# matrix-state linear recurrences (gated linear attention, gated delta rule)
+# ----------------------------------------------------------------------------------------------
+def matrix_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tensor, a_bias: torch.Tensor,
+                state: torch.Tensor, cu: torch.Tensor, slot: torch.Tensor, pos: torch.Tensor, heads: int, kv_heads: int,
+                dim: int, vdim: int, mode: str, tau: float = 1.0, A_log: Optional[torch.Tensor] = None,
+                beta: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Token-by-token f32 recurrence over a [dim, vdim] state per head (``state`` f32
+    [slots, H, dim, vdim], read unless the segment starts at position 0, then replaced), with one
+    decay per head and key channel acting on the state's rows.  ``q``/``k`` [T, G*dim], ``v``
+    [T, H*vdim] (column slices; head h reads q/k head h // (H/G)), ``a`` f32 [T, H*dim] the decay's
+    pre-activation, ``a_bias`` f32 [H*dim].
+
+    ``mode="gla"``:   g = sigmoid(a + a_bias)^(1/tau);  S <- g S + k v^T;  o = S^T (q dim^-1/2).
+    ``mode="delta"``: q, k <- unit vectors (x / sqrt(sum x^2 + 1e-6)), q scaled by dim^-1/2;
+                      g = exp(-exp(A_log[h]) softplus(a + a_bias));  b = sigmoid(beta[t, h]);
+                      S <- g S;  u = b (v - S^T k);  S <- S + k u^T;  o = S^T q.
+    Returns o f32 [T, H*vdim]."""
+    T = q.shape[0]
+    H, G, D, P = heads, kv_heads, dim, vdim
+    S = cu.numel() - 1
+    delta = mode == "delta"
+    assert a.dtype == torch.float32 and a.shape[1] == H * D and q.shape[1] == G * D and v.shape[1] == H * P
+    assert q.dtype == k.dtype == v.dtype
+    if N.use_native(q):
+        out = torch.empty((T, H * P), dtype=torch.float32, device=q.device)
+        N.mcall("mx_matrix_scan", N.ptr(_rows(q)), q.stride(0), N.ptr(_rows(k)), k.stride(0), N.ptr(_rows(v)), v.stride(0),
+                _dt(q), N.ptr(_rows(a)), a.stride(0), N.ptr(a_bias), N.ptr(A_log) if delta else None,
+                N.ptr(_rows(beta)) if delta else None, beta.stride(0) if delta else 0, _dt(beta) if delta else 1,
+                float(tau), 1 if delta else 0, N.ptr(state), N.ptr(cu), N.ptr(slot), N.ptr(pos), N.ptr(out), S, H, G, D, P,
+                N.stream())
+        return out
+    out = torch.zeros((T, H * P), dtype=torch.float32)
+    cul, sll, pl = cu.tolist(), slot.tolist(), pos.tolist()
+    rep = H // G
+    for s in range(S):
+        r0, r1 = cul[s], cul[s + 1]
+        if sll[s] < 0 or r1 <= r0:
+            continue
+        n = r1 - r0
+        qq = q[r0:r1].float().view(n, G, D)
+        kk = k[r0:r1].float().view(n, G, D)
+        vv = v[r0:r1].float().view(n, H, P)
+        z = a[r0:r1].float() + a_bias.float()
+        if delta:
+            qq = qq * torch.rsqrt(qq.pow(2).sum(-1, keepdim=True) + 1e-6)
+            kk = kk * torch.rsqrt(kk.pow(2).sum(-1, keepdim=True) + 1e-6)
+            g = torch.exp(-torch.exp(A_log.float()).repeat_interleave(D)[None] * F.softplus(z)).view(n, H, D)
+            bt = torch.sigmoid(beta[r0:r1].float())
+        else:
+            g = torch.exp(-F.softplus(-z) / tau).view(n, H, D)
+        qq = (qq * D ** -0.5).repeat_interleave(rep, 1)
+        kk = kk.repeat_interleave(rep, 1)
+        St = torch.zeros((H, D, P)) if pl[r0] == 0 else state[sll[s]].clone()
+        for t in range(n):
+            St = g[t][:, :, None] * St
+            u = vv[t]
+            if delta:
+                u = bt[t][:, None] * (u - torch.einsum("hdp,hd->hp", St, kk[t]))
+            St = St + kk[t][:, :, None] * u[:, None, :]
+            out[r0 + t] = torch.einsum("hdp,hd->hp", St, qq[t]).reshape(-1)
+        state[sll[s]] = St
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, w: torch.Tensor, eps: float, gate: torch.Tensor, heads: int, act: str,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """Every head's part of ``o`` [T, H*P] divided by its root mean square over P, times ``w`` [P]
+    (shared by the heads), times act(gate) [T, H*P]; ``act``: sigmoid | silu."""
+    T, n = o.shape
+    P = n // heads
+    if N.use_native(o):
+        out = torch.empty((T, n), dtype=out_dtype, device=o.device)
+        N.mcall("mx_head_norm_gate", N.ptr(_rows(o)), o.stride(0), _dt(o), N.ptr(w), float(eps), N.ptr(_rows(gate)),
+                gate.stride(0), _dt(gate), ACTS[act], N.ptr(out), _dt(out), T, heads, P, N.stream())
+        return out
+    v = o.float().view(T, heads, P)
+    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    return (v.reshape(T, n) * _act(gate.float(), act)).to(out_dtype)
+
+
+# ----------------------------------------------------------------------------------------------
+# real-gated linear recurrent unit
+# ----------------------------------------------------------------------------------------------
+def lru_scan(u: torch.Tensor, z: torch.Tensor, blocks: int, r_bias: torch.Tensor, i_bias: torch.Tensor,
+             lam: torch.Tensor, y: torch.Tensor, y_bias: Optional[torch.Tensor], state: torch.Tensor, cu: torch.Tensor,
+             slot: torch.Tensor, pos: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """Per channel, f32: r = sigmoid(zr + r_bias), i = sigmoid(zi + i_bias), a = exp(-8 r softplus(lam)),
+    S <- a S + sqrt(1 - a^2) i u (also for a sequence's first token, from S = 0); returns
+    S * gelu_tanh(y + y_bias) in ``out_dtype``.  ``u`` f32 [T, R]; ``z`` f32 [blocks, T, 2 * R / blocks]:
+    block b's gate pre-activations [zr | zi] as the batched block-diagonal product leaves them;
+    ``y`` a column slice; ``state`` f32 [slots, R], read unless the segment starts at position 0,
+    then replaced."""
+    T, R = u.shape
+    S = cu.numel() - 1
+    bs = R // blocks
+    assert u.dtype == z.dtype == torch.float32 and u.is_contiguous() and z.is_contiguous()
+    assert tuple(z.shape) == (blocks, T, 2 * bs)
+    if N.use_native(u):
+        out = torch.empty((T, R), dtype=out_dtype, device=u.device)
+        N.mcall("mx_lru_scan", N.ptr(u), N.ptr(z), blocks, N.ptr(r_bias), N.ptr(i_bias), N.ptr(lam), N.ptr(_rows(y)),
+                y.stride(0), _dt(y), N.ptr(y_bias), N.ptr(state), N.ptr(cu), N.ptr(slot), N.ptr(pos), N.ptr(out), _dt(out),
+                S, R, T, N.stream())
+        return out
+    zr = z[:, :, :bs].transpose(0, 1).reshape(T, R)
+    zi = z[:, :, bs:].transpose(0, 1).reshape(T, R)
+    out = torch.zeros((T, R), dtype=torch.float32)
+    cul, sll, pl = cu.tolist(), slot.tolist(), pos.tolist()
+    a = torch.exp(-8.0 * torch.sigmoid(zr + r_bias.float()) * F.softplus(lam.float()))
+    bx = torch.sqrt(1.0 - a * a) * torch.sigmoid(zi + i_bias.float()) * u
+    yy = y.float() + (y_bias.float() if y_bias is not None else 0.0)
+    for s in range(S):
+        r0, r1 = cul[s], cul[s + 1]
+        if sll[s] < 0 or r1 <= r0:
+            continue
+        St = torch.zeros(R) if pl[r0] == 0 else state[sll[s]].clone()
+        for t in range(r0, r1):
+            St = a[t] * St + bx[t]
+            out[t] = St
+        state[sll[s]] = St
+    return (out * F.gelu(yy, approximate="tanh")).to(out_dtype)
+
+
+# ----------------------------------------------------------------------------------------------
+# sliding-window attention with grouped key/value heads over a paged row cache
+# ----------------------------------------------------------------------------------------------
+def qk_norm_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qw: Optional[torch.Tensor],
+                  kw: Optional[torch.Tensor], eps: float, slots: torch.Tensor, cache: torch.Tensor) -> torch.Tensor:
+    """Per token: RMS norm of the WHOLE query projection (all heads at once) times ``qw`` -> returned
+    [T, nq]; the same for the key projection with ``kw``; the normed keys and the values go to cache
+    row ``slots[t]`` as [k | v] (< 0: no write).  ``qw``/``kw`` None: no norm."""
+    T, nq = q.shape
+    nk, nv = k.shape[1], v.shape[1]
+    assert cache.shape[-1] == nk + nv
+    if N.use_native(q):
+        assert q.dtype == k.dtype == v.dtype == cache.dtype
+        out = torch.empty((T, nq), dtype=q.dtype, device=q.device)
+        N.mcall("mx_qk_norm_write", N.ptr(_rows(q)), q.stride(0), N.ptr(_rows(k)), k.stride(0), N.ptr(_rows(v)), v.stride(0),
+                N.ptr(qw), N.ptr(kw), float(eps), N.ptr(slots), N.ptr(cache), N.ptr(out), _dt(q), T, nq, nk, nv, N.stream())
+        return out
+    rms = lambda t, w: (t.float() * torch.rsqrt(t.float().pow(2).mean(-1, keepdim=True) + eps) * w.float()  # noqa: E731
+                        if w is not None else t.float())
+    rows = torch.cat([rms(k, kw), v.float()], 1).to(cache.dtype)
+    ok = slots >= 0
+    cache.view(-1, nk + nv)[slots[ok].long()] = rows[ok]
+    return rms(q, qw).to(q.dtype)
+
+
+def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: torch.Tensor, bt: torch.Tensor,
+                  window: int, scale: float, max_len: int, heads: int, kv_heads: int, dim: int, vdim: int,
+                  gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal softmax attention of ``q`` [T, H*dim] over the cache rows [k: G*dim | v: G*vdim] of each
+    segment's pages: the query at position p sees keys j with 0 <= p - j < window; query head h
+    reads key/value head h // (H/G); score = q . k * scale, f32 softmax; head h's output is
+    multiplied by sigmoid(gate[t, h]) when a gate [T, H] is given.  Returns [T, H*vdim]."""
+    T = q.shape[0]
+    H, G, D, P = heads, kv_heads, dim, vdim
+    S = cu.numel() - 1
+    Wr = G * (D + P)
+    if N.use_native(q):
+        assert bt.is_contiguous() and q.dtype == cache.dtype
+        out = torch.empty((T, H * P), dtype=q.dtype, device=q.device)
+        N.mcall("mx_window_attend", N.ptr(_rows(q)), q.stride(0), N.ptr(cache), N.ptr(cu), N.ptr(pos), N.ptr(bt), bt.shape[1],
+                N.ptr(_rows(gate)) if gate is not None else None, gate.stride(0) if gate is not None else 0,
+                int(min(window, 1 << 30)), float(scale), N.ptr(out), _dt(q), S, int(max_len), H, G, D, P, N.stream())
+        return out
+    out = torch.zeros((T, H, P), dtype=torch.float32)
+    rows = cache.view(-1, Wr).float()
+    cul, pl = cu.tolist(), pos.tolist()
+    rep = H // G
+    for s in range(S):
+        a, b = cul[s], cul[s + 1]
+        if b <= a:
+            continue
+        ctx = pl[b - 1] + 1
+        pages = bt[s, :(ctx + PAGE - 1) // PAGE].long()
+        kv = rows.view(-1, PAGE, Wr)[pages].reshape(-1, Wr)[:ctx]
+        keys = kv[:, :G * D].view(ctx, G, D).repeat_interleave(rep, 1)
+        vals = kv[:, G * D:].view(ctx, G, P).repeat_interleave(rep, 1)
+        sc = torch.einsum("nhd,jhd->nhj", q[a:b].float().view(-1, H, D), keys) * scale
+        p = pos[a:b].long()[:, None]
+        j = torch.arange(ctx)[None]
+        vis = (j <= p) & (j > p - window)
+        sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
+        out[a:b] = torch.einsum("nhj,jhp->nhp", torch.softmax(sc, -1), vals)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())[:, :, None]
+    return out.reshape(T, H * P).to(q.dtype)
