@@ -186,3 +186,13 @@ def forward(cfg: Dict, sd: Dict[str, torch.Tensor], tokens: List[int], streams: 
         if streams is not None:
             streams.append(x.clone())
     return layer_norm(x, sd["final.norm"].to(F64), eps) @ sd["head"].to(F64).T
+
+
+def greedy(cfg: Dict, sd: Dict[str, torch.Tensor], prompt: List[int], n: int) -> List[int]:
+    """``n`` greedy tokens after ``prompt``, each from a whole-sequence forward pass."""
+    toks, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(forward(cfg, sd, toks)[-1].argmax())
+        out.append(nxt)
+        toks.append(nxt)
+    return out
