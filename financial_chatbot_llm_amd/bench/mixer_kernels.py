@@ -1,12 +1,15 @@
 """Times the sequence-mixer kernels (``ops.mixers``) at the layer shapes of a hybrid decoder.
 
-    python -m financial_chatbot_llm_amd.bench.mixer_kernels [--width 2048]
+    python -m financial_chatbot_llm_amd.bench.mixer_kernels [--width 2048] [--design gezavik|sigudra]
 
 Two step shapes: a prefill step of two 2048-token prompts and a decode step of 64 single rows at
 depth 1024.  Shapes follow ``models.gezavik.example_config(scale_up=True)``: Mamba-2 with inner =
 2 * width, 64-wide heads, state 128, 2 groups, 4 taps; latent attention with width / 128 heads,
 kv_rank 256, rot_dim 32, window 1024.  One JSON line per kernel and shape (microseconds, and the
-arithmetic or byte rate the time corresponds to).
+arithmetic or byte rate the time corresponds to).  ``--design sigudra``: the kernels of that design at
+``models.sigudra.example_config(scale_up=True)`` shapes (width / 128 heads of key and value size 128
+for the delta rule and the windowed attention with 4 query heads per key/value head, 64-wide keys for
+gated linear attention, a gated LRU as wide as the model, window 1024).
 """
 from __future__ import annotations
 
@@ -31,10 +34,93 @@ def _time(f, n: int = 20) -> float:
     return a.elapsed_time(b) / n * 1e3
 
 
+def _steps(dev):
+    for name, lens, start in (("prefill 2x2048", [2048, 2048], 0), ("decode 64x1 at 1024", [1] * 64, 1024)):
+        cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32, device=dev)
+        pos = torch.cat([torch.arange(start, start + n) for n in lens]).to(torch.int32).to(dev)
+        yield name, lens, start, cu, pos, torch.arange(len(lens), dtype=torch.int32, device=dev)
+
+
+def sigudra(width: int) -> int:
+    dev = "cuda"
+    H, D, P, K, window = max(width // 128, 2), 128, 128, 4, 1024
+    G = max(H // 4, 1)
+    out = lambda **kw: print(json.dumps(kw), flush=True)  # noqa: E731
+    for name, lens, start, cu, pos, slot in _steps(dev):
+        S, T, ml = len(lens), sum(lens), max(lens)
+        # delta rule: convolution over q | k | v, then the scan
+        C = 2 * H * D + H * P
+        inp = torch.randn(T, C, device=dev).bfloat16()
+        cw = torch.randn(C, K, device=dev)
+        cst = torch.zeros(S, K - 1, C, device=dev)
+        us = _time(lambda: mx.conv_act(inp, cw, None, cst, cu, slot, pos, ml, "silu"))
+        out(shape=name, kernel="conv_act", us=round(us, 1), TB_per_s=round(T * C * 6 / us / 1e6, 2))
+        u = mx.conv_act(inp, cw, None, cst, cu, slot, pos, ml, "silu")
+        a_ = torch.randn(T, H * D, device=dev)
+        ab, Al = torch.zeros(H * D, device=dev), torch.zeros(H, device=dev)
+        beta = torch.randn(T, H, device=dev).bfloat16()
+        st = torch.zeros(S, H, D, P, device=dev)
+        nq = H * D
+        us = _time(lambda: mx.matrix_scan(u[:, :nq], u[:, nq:2 * nq], u[:, 2 * nq:], a_, ab, st, cu, slot, pos, H, H, D, P,
+                                          "delta", A_log=Al, beta=beta), 5)
+        out(shape=name, kernel="matrix_scan delta", us=round(us, 1), f32_TFLOP_per_s=round(T * H * D * P * 9 / us / 1e6, 2),
+            state_TB_per_s=round(S * H * D * P * 8 / us / 1e6, 2))
+        Dg = 64
+        qkv = torch.randn(T, 2 * H * Dg + H * P, device=dev).bfloat16() * 0.1
+        ag = torch.randn(T, H * Dg, device=dev) + 3
+        stg = torch.zeros(S, H, Dg, P, device=dev)
+        us = _time(lambda: mx.matrix_scan(qkv[:, :H * Dg], qkv[:, H * Dg:2 * H * Dg], qkv[:, 2 * H * Dg:], ag,
+                                          ab[:H * Dg], stg, cu, slot, pos, H, H, Dg, P, "gla", tau=16.0), 5)
+        out(shape=name, kernel="matrix_scan gla", us=round(us, 1), f32_TFLOP_per_s=round(T * H * Dg * P * 5 / us / 1e6, 2),
+            state_TB_per_s=round(S * H * Dg * P * 8 / us / 1e6, 2))
+        o = torch.randn(T, H * P, device=dev)
+        gt = torch.randn(T, H * P, device=dev).bfloat16()
+        nw = torch.ones(P, device=dev)
+        us = _time(lambda: mx.head_norm_gate(o, nw, 1e-5, gt, H, "sigmoid", torch.bfloat16))
+        out(shape=name, kernel="head_norm_gate", us=round(us, 1), TB_per_s=round(T * H * P * 8 / us / 1e6, 2))
+        # gated LRU
+        R, Bk = width, max(width // 256, 1)
+        uu = torch.randn(T, R, device=dev)
+        z = torch.randn(Bk, T, 2 * R // Bk, device=dev)
+        rb, lam = torch.zeros(R, device=dev), torch.zeros(R, device=dev)
+        y = torch.randn(T, R, device=dev).bfloat16()
+        sl = torch.zeros(S, R, device=dev)
+        us = _time(lambda: mx.lru_scan(uu, z, Bk, rb, rb, lam, y, rb, sl, cu, slot, pos, torch.bfloat16))
+        out(shape=name, kernel="lru_scan", us=round(us, 1), TB_per_s=round(T * R * 16 / us / 1e6, 2))
+        # windowed attention
+        pages = (start + ml + 63) // 64
+        cache = torch.randn(S * pages * 64, G * (D + P), device=dev).bfloat16()
+        bt = torch.arange(S * pages, dtype=torch.int32, device=dev).view(S, pages).contiguous()
+        q = torch.randn(T, H * D, device=dev).bfloat16() * .1
+        k = torch.randn(T, G * D, device=dev).bfloat16()
+        v = torch.randn(T, G * P, device=dev).bfloat16()
+        qw, kw = torch.ones(H * D, device=dev), torch.ones(G * D, device=dev)
+        slots = (bt[:, None, :].expand(S, ml, pages).reshape(-1, pages).gather(1, (pos // 64).long()[:, None])[:, 0] * 64
+                 + pos % 64).to(torch.int32)
+        us = _time(lambda: mx.qk_norm_write(q, k, v, qw, kw, 1e-5, slots, cache))
+        out(shape=name, kernel="qk_norm_write", us=round(us, 1),
+            TB_per_s=round(T * (2 * H * D + 2 * G * (D + P)) * 2 / us / 1e6, 2))
+        gate = torch.randn(T, H, device=dev).bfloat16()
+        us = _time(lambda: mx.window_attend(q, cache, cu, pos, bt, window, 0.1, ml, H, G, D, P, gate=gate), 5)
+        pairs = sum(min(p + 1, window) for n in lens for p in range(start, start + n))
+        out(shape=name, kernel="window_attend", us=round(us, 1),
+            bf16_TFLOP_per_s=round(pairs * H * 2 * (D + P) / us / 1e6, 1),
+            cache_TB_per_s=round(S * min(start + ml, window + ml) * G * (D + P) * 2 / us / 1e6, 2))
+        x = torch.randn(T, width, device=dev)
+        aa = torch.randn(T, width, device=dev).bfloat16()
+        w = torch.ones(width, device=dev)
+        us = _time(lambda: mx.post_norm_add(x, aa, w, 1e-5, torch.bfloat16))
+        out(shape=name, kernel="post_norm_add", us=round(us, 1), TB_per_s=round(T * width * 12 / us / 1e6, 2))
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--width", type=int, default=2048)
+    ap.add_argument("--design", default="gezavik", choices=["gezavik", "sigudra"])
     a = ap.parse_args(argv)
+    if a.design == "sigudra":
+        return sigudra(a.width)
     dev = "cuda"
     H, P, Ns, G, K = 2 * a.width // 64, 64, 128, 2, 4
     C = H * P + 2 * G * Ns

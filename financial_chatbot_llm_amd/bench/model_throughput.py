@@ -1,7 +1,8 @@
 """Prefill and decode throughput of a layered hybrid decoder beside a Llama twin of equal size.
 
     python bench.py --model-throughput gezavik [--mt-widths 1024,2048,4096]
-    python -m financial_chatbot_llm_amd.bench.model_throughput --only gezavik-w2048
+    python bench.py --model-throughput sigudra          # beside Gezavik, its closest relative here
+    python -m financial_chatbot_llm_amd.bench.model_throughput --mt-only gezavik-w2048
 
 For each width a Gezavik model (random weights, 8 layers: latent attention and Mamba-2 mixers, dense
 and routed feed-forwards, sizes in the range of a real model's layers) and a Llama model of the same
@@ -70,6 +71,17 @@ def register(width: int, vocab: int = 32768) -> List[str]:
     REGISTRY[l] = ModelConfig(l, "llama", vocab, width, L, heads, kvh, 128, ff, max_position=8192,
                               bos_token_id=0, eos_token_ids=())
     return [g, l]
+
+
+def register_sigudra(width: int, vocab: int = 32768) -> List[str]:
+    """Register ``sigudra-w<width>`` (8 layers ``dGPgDpdG``: delta rule, gated linear attention and
+    windowed attention beside a gated LRU; dense and routed feed-forwards) and the Gezavik model of the
+    same width, depth and vocabulary; returns the two names."""
+    from ..models.configs import REGISTRY, layered_config
+    from ..models.sigudra import example_config
+    name = f"sigudra-w{width}"
+    REGISTRY[name] = layered_config(example_config(width=width, vocab=vocab, pattern="dGPgDpdG", scale_up=True), name)
+    return [name, register(width, vocab)[0]]
 
 
 def _tokens(n: int, vocab: int, seed: int) -> List[int]:
@@ -141,8 +153,9 @@ def add_arguments(ap: argparse.ArgumentParser) -> None:
 
 def run(a) -> int:
     names: List[str] = []
+    design = getattr(a, "model_throughput", "") or "gezavik"
     for w in (int(x) for x in a.mt_widths.split(",") if x):
-        names += register(w)
+        names += register_sigudra(w) if design == "sigudra" else register(w)
     if a.mt_only:
         names = [n for n in names if n == a.mt_only]
     for n in names:
@@ -153,6 +166,7 @@ def run(a) -> int:
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--model-throughput", default="gezavik", choices=["gezavik", "sigudra"])
     add_arguments(ap)
     return run(ap.parse_args(argv))
 

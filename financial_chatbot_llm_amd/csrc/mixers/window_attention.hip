@@ -178,7 +178,276 @@ window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cac
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// bf16 on the matrix cores (v_mfma_f32_16x16x32_bf16).  A block owns 64 (row, head) pairs of one
+// segment and ONE key/value head -- QT consecutive rows x HB of its query heads, 16 pairs per wave --
+// and walks the key tiles of the union of their windows, KT = 32 keys at a time.  Per tile and wave:
+//     S^T = K . Q^T      A: key rows from LDS (16-byte reads), B: the wave's queries, in registers
+//     online softmax     the statistics of query (lane % 16) live in that lane, f32
+//     O^T += V^T . P^T   A: the value tile, transposed in LDS; B: P straight from the S^T registers
+//                        (the MFMA's k slots 8g+i / 8g+4+i hold keys 4g+i / 16+4g+i)
+// Feature dimensions are zero-padded to multiples of 32 (keys) / 16 (values) in LDS and registers.
+// Single-row segments (decode) may split each row's key range over nsplit blocks; the parts
+// (unnormalised output, running maximum, sum) are combined by window_merge_kernel.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int MKT = 32;             // keys per tile
+constexpr int MLDV = MKT + 8;       // row stride of the transposed value tile
+
+template <int KSM, int NTM>         // up to 32*KSM key dims, 16*NTM value dims
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __restrict__ cache,
+                          const int* __restrict__ cu, const int* __restrict__ pos, const int* __restrict__ bt, int btw,
+                          const bf16* __restrict__ gate, long sgate, int window, float scale, bf16* __restrict__ out,
+                          int H, int G, int D, int P, int QT, int HB, int nsplit, float* __restrict__ ws) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int KS = (D + 31) / 32, NT = (P + 15) / 16;
+  const int ldk = KS * 32 + 8;
+  bf16* kt_lds = reinterpret_cast<bf16*>(smem);                 // [MKT][ldk]
+  bf16* vt_lds = kt_lds + MKT * ldk;                            // [NT*16][MLDV]
+  const int rep = H / G;
+  const int hblocks = (rep + HB - 1) / HB;
+  const int s = blockIdx.z;
+  const int r0 = cu[s], n = cu[s + 1] - r0;
+  // nsplit > 1 (single-row segments): blockIdx.x is the part of the key range this block walks
+  const int split = nsplit > 1 ? blockIdx.x : 0;
+  const int t0 = nsplit > 1 ? 0 : blockIdx.x * QT;
+  if (t0 >= n) return;
+  const int nq = min(QT, n - t0);
+  const int kvh = blockIdx.y / hblocks;
+  const int hg0 = (blockIdx.y - kvh * hblocks) * HB;
+  const int nh = min(HB, rep - hg0);
+  const int h0 = kvh * rep + hg0;
+  const int Wr = G * (D + P);
+  const int koff = kvh * D, voff = G * D + kvh * P;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
+  const int p_first = pos[r0 + t0], p_last = pos[r0 + t0 + nq - 1];
+  const int lo = max(0, p_first - window + 1);
+  // this lane's query: pair index 16 * wave + c
+  const int pair = 16 * wave + c;
+  const bool qok = pair < nq * nh;
+  const int tq = qok ? pair / nh : 0, hh = qok ? pair - (pair / nh) * nh : 0;
+  const long row = r0 + t0 + tq;
+  const int h = h0 + hh;
+  const int pq = qok ? pos[row] : -1;
+  const bool wave_live = 16 * wave < nq * nh;
+
+  bf16x8 qf[KSM];
+#pragma unroll
+  for (int ks = 0; ks < KSM; ++ks) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int d = 32 * ks + 8 * g + e;
+      qf[ks][e] = (qok && d < D) ? q[row * sq + (long)h * D + d] : (bf16)0.f;
+    }
+  }
+  f32x4 o[NTM];
+#pragma unroll
+  for (int nt = 0; nt < NTM; ++nt) o[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  // zero the padding columns / rows once (staging only writes real elements)
+  if ((D & 31) != 0 || (P & 15) != 0) {
+    unsigned* z = reinterpret_cast<unsigned*>(smem);
+    const int words = (MKT * ldk + NT * 16 * MLDV) / 2;
+    for (int e = threadIdx.x; e < words; e += 256) z[e] = 0u;
+  }
+
+  int k_begin = (lo / MKT) * MKT, k_end = p_last;     // first tile start, last key
+  if (nsplit > 1) {
+    const int tiles = (p_last - k_begin) / MKT + 1;
+    const int per = (tiles + nsplit - 1) / nsplit;
+    k_begin += split * per * MKT;
+    k_end = min(p_last, k_begin + per * MKT - 1);
+  }
+  // staging, 16-byte path (D, P multiples of 8): a work item is a pair of keys x 8 dims of the key
+  // part or of the value part -- two row loads; key pieces go to the key tile as two 16-byte stores,
+  // value pieces to the transposed value tile as eight 4-byte stores (one key pair each).  The next
+  // tile's loads are issued before the current tile's MFMAs and land in registers while they run.
+  constexpr int MAXIT = (KSM * 32 + NTM * 16) / 8 * 16 / 256;      // 16 pairs * pieces / 256 threads
+  const bool v16 = (D & 7) == 0 && (P & 7) == 0;
+  const int dk8 = D >> 3, d8 = (D + P) >> 3;
+  bf16x8 pre[MAXIT][2];
+  auto load_tile = [&](int k0) {
+    const int rows = min(MKT, p_last + 1 - k0);
+    const bf16* src = cache + ((long)bt[(long)s * btw + k0 / PAGE] * PAGE + (k0 % PAGE)) * Wr;
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int e = min((int)threadIdx.x + 256 * it, 16 * d8 - 1);
+      const int piece = e >> 4, jp = e & 15;
+      const int col = piece < dk8 ? koff + piece * 8 : voff + (piece - dk8) * 8;
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int j = 2 * jp + r;
+        bf16x8 v = *reinterpret_cast<const bf16x8*>(src + (long)min(j, rows - 1) * Wr + col);
+        if (j >= rows)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[i] = (bf16)0.f;
+        pre[it][r] = v;
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int it = 0; it < MAXIT; ++it) {
+      const int e = threadIdx.x + 256 * it;
+      if (e < 16 * d8) {
+        const int piece = e >> 4, jp = e & 15;
+        if (piece < dk8) {
+          *reinterpret_cast<bf16x8*>(kt_lds + (2 * jp) * ldk + piece * 8) = pre[it][0];
+          *reinterpret_cast<bf16x8*>(kt_lds + (2 * jp + 1) * ldk + piece * 8) = pre[it][1];
+        } else {
+          const int d = (piece - dk8) * 8;
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            *reinterpret_cast<bf16x2*>(vt_lds + (d + i) * MLDV + 2 * jp) = bf16x2{pre[it][0][i], pre[it][1][i]};
+        }
+      }
+    }
+  };
+  if (v16 && k_begin <= k_end) load_tile(k_begin);
+  for (int k0 = k_begin; k0 <= k_end; k0 += MKT) {
+    __syncthreads();
+    const int rows = min(MKT, p_last + 1 - k0);
+    if (v16) {
+      store_tile();
+    } else {
+      const bf16* src = cache + ((long)bt[(long)s * btw + k0 / PAGE] * PAGE + (k0 % PAGE)) * Wr;
+      for (int e = threadIdx.x; e < MKT * D; e += 256) {
+        const int j = e / D, d = e - j * D;
+        kt_lds[j * ldk + d] = j < rows ? src[(long)j * Wr + koff + d] : (bf16)0.f;
+      }
+      for (int e = threadIdx.x; e < MKT * P; e += 256) {
+        const int j = e / P, d = e - j * P;
+        vt_lds[d * MLDV + j] = j < rows ? src[(long)j * Wr + voff + d] : (bf16)0.f;
+      }
+    }
+    __syncthreads();
+    if (v16 && k0 + MKT <= k_end) load_tile(k0 + MKT);
+    if (!wave_live) continue;
+    // S^T for the two 16-key halves
+    f32x4 st[2];
+    float sc[2][4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh) {
+      st[kh] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16* kr = kt_lds + (16 * kh + c) * ldk + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < KSM; ++ks)
+        if (ks < KS) st[kh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(kr + 32 * ks), qf[ks], st[kh], 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = k0 + 16 * kh + 4 * g + i;
+        const bool vis = j <= pq && j > pq - window;
+        sc[kh][i] = vis ? st[kh][i] * scale : -INFINITY;
+        tmax = fmaxf(tmax, sc[kh][i]);
+      }
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float mn = fmaxf(m, tmax);
+    const float corr = (m == -INFINITY) ? 0.f : expf(m - mn);
+    bf16x8 pb;
+    float psum = 0.f;
+#pragma unroll
+    for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = sc[kh][i] == -INFINITY ? 0.f : expf(sc[kh][i] - mn);
+        psum += p;
+        pb[4 * kh + i] = (bf16)p;
+      }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = mn;
+#pragma unroll
+    for (int nt = 0; nt < NTM; ++nt) {
+      if (nt < NT) {
+        const bf16* vr = vt_lds + (16 * nt + c) * MLDV + 4 * g;
+        const bf16x4 a0 = *reinterpret_cast<const bf16x4*>(vr), a1 = *reinterpret_cast<const bf16x4*>(vr + 16);
+        bf16x8 a;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          a[i] = a0[i];
+          a[4 + i] = a1[i];
+        }
+        o[nt] *= corr;
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[nt], 0, 0, 0);
+      }
+    }
+  }
+  if (!qok) return;
+  if (nsplit > 1) {                          // unnormalised part: o | m | l, merged by window_merge_kernel
+    float* w = ws + ((row * H + h) * nsplit + split) * (long)(P + 2);
+#pragma unroll
+    for (int nt = 0; nt < NTM; ++nt)
+      if (nt < NT)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = 16 * nt + 4 * g + i;
+          if (r < P) w[r] = o[nt][i];
+        }
+    if (g == 0) {
+      w[P] = m;
+      w[P + 1] = l;
+    }
+    return;
+  }
+  float gsc = 1.0f / l;
+  if (gate != nullptr) gsc *= mx_sigmoid((float)gate[row * sgate + h]);
+  bf16* dst = out + (row * H + h) * P;
+#pragma unroll
+  for (int nt = 0; nt < NTM; ++nt) {
+    if (nt < NT) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * nt + 4 * g + i;
+        if (r < P) dst[r] = (bf16)(o[nt][i] * gsc);
+      }
+    }
+  }
+}
+
+// grid (rows, H): combine the nsplit parts of one (row, head)
+__global__ void window_merge_kernel(const float* __restrict__ ws, const bf16* __restrict__ gate, long sgate,
+                                    bf16* __restrict__ out, int H, int P, int nsplit) {
+  const long row = blockIdx.x;
+  const int h = blockIdx.y;
+  const float* w = ws + (row * H + h) * nsplit * (long)(P + 2);
+  float M = -INFINITY;
+  for (int i = 0; i < nsplit; ++i) M = fmaxf(M, w[i * (P + 2) + P]);
+  float L = 0.f;
+  for (int i = 0; i < nsplit; ++i) {
+    const float mi = w[i * (P + 2) + P];
+    if (mi != -INFINITY) L += w[i * (P + 2) + P + 1] * expf(mi - M);
+  }
+  float gsc = 1.0f / L;
+  if (gate != nullptr) gsc *= mx_sigmoid((float)gate[row * sgate + h]);
+  for (int r = threadIdx.x; r < P; r += blockDim.x) {
+    float a = 0.f;
+    for (int i = 0; i < nsplit; ++i) {
+      const float mi = w[i * (P + 2) + P];
+      if (mi != -INFINITY) a += w[i * (P + 2) + r] * expf(mi - M);
+    }
+    out[(row * H + h) * P + r] = (bf16)(a * gsc);
+  }
+}
+
 }  // namespace
+
+// MX_ATTEND_MFMA=0 keeps every call on the f32-lane kernel (A/B and debugging)
+static bool wa_use_mfma() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("MX_ATTEND_MFMA");
+    v = (e != nullptr && e[0] == '0') ? 0 : 1;
+  }
+  return v == 1;
+}
 
 // q [T, nq], k [T, nk], v [T, nv] slices (row strides sq, sk, sv); qw [nq], kw [nk] f32 (null: no norm);
 // cache [pages*64, nk + nv]; qout [T, nq] contiguous; all of storage type dt
@@ -193,12 +462,36 @@ MX_API int mx_qk_norm_write(const void* q, long sq, const void* k, long sk, cons
 
 // q [T, H*D] (row stride sq), out [T, H*P] contiguous; cu [S+1] row bounds of the segments, pos [T]
 // positions, bt [S, btw] page tables; gate [T, >= H] slice (row stride sgate) or null.
+// nsplit > 1 with a workspace ws (f32 [T, H, nsplit, P + 2]) and single-row segments: the key range of
+// each row is walked by nsplit blocks and merged (bf16 matrix-core form only; ignored otherwise).
 MX_API int mx_window_attend(const void* q, long sq, const void* cache, const int* cu, const int* pos, const int* bt,
                             int btw, const void* gate, long sgate, int window, float scale, void* out, int dt, int S,
-                            int max_len, int H, int G, int D, int P, hipStream_t st) {
+                            int max_len, int H, int G, int D, int P, int nsplit, float* ws, hipStream_t st) {
   if (S <= 0 || max_len <= 0) return 0;
   if (P > 64 * WA_CPL || G < 1 || H % G || window < 1) return (int)hipErrorInvalidValue;
   const int rep = H / G;
+  if (dt == 0 && D <= 256 && P <= 256 && wa_use_mfma()) {
+    // matrix-core form: 64 (row, head) pairs of one key/value head per block
+    const int HB = rep < 64 ? rep : 64;
+    const int QT = max_len == 1 ? 1 : (64 / HB > 0 ? 64 / HB : 1);
+    const int KS = (D + 31) / 32, NT = (P + 15) / 16;
+    const size_t lds = ((size_t)MKT * (KS * 32 + 8) + (size_t)NT * 16 * MLDV) * sizeof(bf16);
+    if (max_len != 1 || ws == nullptr || nsplit < 1) nsplit = 1;
+    dim3 grid(nsplit > 1 ? nsplit : (max_len + QT - 1) / QT, G * ((rep + HB - 1) / HB), S);
+    if (D <= 128 && P <= 128)
+      window_attend_mfma_kernel<4, 8><<<grid, 256, lds, st>>>(
+          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, scale, (bf16*)out, H,
+          G, D, P, QT, HB, nsplit, ws);
+    else
+      window_attend_mfma_kernel<8, 16><<<grid, 256, lds, st>>>(
+          (const bf16*)q, sq, (const bf16*)cache, cu, pos, bt, btw, (const bf16*)gate, sgate, window, scale, (bf16*)out, H,
+          G, D, P, QT, HB, nsplit, ws);
+    if (nsplit > 1) {
+      dim3 g2(S, H);           // single-row segments: row index == segment index
+      window_merge_kernel<<<g2, P >= 128 ? 128 : 64, 0, st>>>(ws, (const bf16*)gate, sgate, (bf16*)out, H, P, nsplit);
+    }
+    MX_RETURN_LAUNCH();
+  }
   const int esz = dt == 1 ? 4 : 2;
   // key row stride: odd in 4-byte words
   int ldk = D;

@@ -667,9 +667,18 @@ def window_attend(q: torch.Tensor, cache: torch.Tensor, cu: torch.Tensor, pos: t
     if N.use_native(q):
         assert bt.is_contiguous() and q.dtype == cache.dtype
         out = torch.empty((T, H * P), dtype=q.dtype, device=q.device)
+        # decode-size steps (one row per segment) walk each row's keys with several blocks so that a
+        # small batch still fills the chip; the split depends only on static sizes (graph-safe)
+        nsplit, ws = 1, None
+        if max_len == 1 and q.dtype == torch.bfloat16:
+            tiles = (min(window, bt.shape[1] * PAGE) + 31) // 32 + 1
+            nsplit = max(1, min(16, tiles // 2, 1024 // max(S * G, 1)))
+            if nsplit > 1:
+                ws = torch.empty((T, H, nsplit, P + 2), dtype=torch.float32, device=q.device)
         N.mcall("mx_window_attend", N.ptr(_rows(q)), q.stride(0), N.ptr(cache), N.ptr(cu), N.ptr(pos), N.ptr(bt), bt.shape[1],
                 N.ptr(_rows(gate)) if gate is not None else None, gate.stride(0) if gate is not None else 0,
-                int(min(window, 1 << 30)), float(scale), N.ptr(out), _dt(q), S, int(max_len), H, G, D, P, N.stream())
+                int(min(window, 1 << 30)), float(scale), N.ptr(out), _dt(q), S, int(max_len), H, G, D, P, nsplit,
+                N.ptr(ws), N.stream())
         return out
     out = torch.zeros((T, H, P), dtype=torch.float32)
     rows = cache.view(-1, Wr).float()
