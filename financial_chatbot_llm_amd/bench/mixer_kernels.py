@@ -62,7 +62,7 @@ def sigudra(width: int) -> int:
         st = torch.zeros(S, H, D, P, device=dev)
         nq = H * D
         us = _time(lambda: mx.matrix_scan(u[:, :nq], u[:, nq:2 * nq], u[:, 2 * nq:], a_, ab, st, cu, slot, pos, H, H, D, P,
-                                          "delta", A_log=Al, beta=beta), 5)
+                                          "delta", A_log=Al, beta=beta, max_len=ml), 5)
         out(shape=name, kernel="matrix_scan delta", us=round(us, 1), f32_TFLOP_per_s=round(T * H * D * P * 9 / us / 1e6, 2),
             state_TB_per_s=round(S * H * D * P * 8 / us / 1e6, 2))
         Dg = 64
@@ -70,7 +70,7 @@ def sigudra(width: int) -> int:
         ag = torch.randn(T, H * Dg, device=dev) + 3
         stg = torch.zeros(S, H, Dg, P, device=dev)
         us = _time(lambda: mx.matrix_scan(qkv[:, :H * Dg], qkv[:, H * Dg:2 * H * Dg], qkv[:, 2 * H * Dg:], ag,
-                                          ab[:H * Dg], stg, cu, slot, pos, H, H, Dg, P, "gla", tau=16.0), 5)
+                                          ab[:H * Dg], stg, cu, slot, pos, H, H, Dg, P, "gla", tau=16.0, max_len=ml), 5)
         out(shape=name, kernel="matrix_scan gla", us=round(us, 1), f32_TFLOP_per_s=round(T * H * Dg * P * 5 / us / 1e6, 2),
             state_TB_per_s=round(S * H * Dg * P * 8 / us / 1e6, 2))
         o = torch.randn(T, H * P, device=dev)

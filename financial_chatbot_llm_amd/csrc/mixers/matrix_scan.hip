@@ -5,15 +5,25 @@
 //     gla:    g = sigmoid(a + a_bias)^(1/tau);              S <- g S + k v^T;            o = S^T q
 //     delta:  g = exp(-exp(A_log[h]) softplus(a + a_bias));  S <- g S;  u = b (v - S^T k);
 //             S <- S + k u^T;  o = S^T q;    q, k unit vectors per head first, b = sigmoid(beta)
-//   and q scaled by D^-1/2 in both.  Column p of S never meets another column, so a lane owns RPL
-//   rows of one column in registers and LPC neighbouring lanes share a column (D <= RPL * LPC); the
-//   two dot products per token are reduced over those lanes with DPP swaps.  The rows of a chunk of
-//   tokens (q, k, the decay, the block's v and b) are staged -- and transformed -- in LDS once per
-//   block; the outputs of the chunk leave through LDS as whole runs.
+//   and q scaled by D^-1/2 in both.  Two launches:
+//     prep   one block per token, fully parallel: the decays g (written over `a`), and for the delta
+//            rule the unit-norm factors of q and k and sigmoid(beta);
+//     scan   column p of S never meets another column, so a lane owns RPL rows of one column in
+//            registers and LPC neighbouring lanes share a column (D <= RPL * LPC); the two dot
+//            products per token are reduced over those lanes with DPP swaps.  The rows of a chunk
+//            of TB tokens (q, k, g, the block's v and b) are staged in LDS once per block; the next
+//            chunk's rows are fetched into registers -- clamped loads, issued back to back -- before
+//            the current chunk's dependent steps run; the chunk's outputs leave through LDS as
+//            whole runs.  Steps with few (segment, head) pairs take the variant with more lanes per
+//            column so that the grid still covers the chip.
 //
 // mx_lru_scan: a diagonal recurrence per channel, S <- a S + sqrt(1 - a^2) i u with
 //     a = exp(-8 sigmoid(zr + r_bias) softplus(lam)),  i = sigmoid(zi + i_bias),
-//   output S * gelu_tanh(y + y_bias).
+//   output S * gelu_tanh(y + y_bias).  Two launches: the gates (a, the input term and the GeLU
+//   branch: every transcendental) elementwise over all rows, then the recurrence itself, where a
+//   block walks 64 tokens at a time: each thread scans 16 tokens of one channel from zero, the four
+//   partial maps S -> A S + B are folded through LDS, and the outputs are corrected by the true
+//   start state.
 #include "mx_common.h"
 
 namespace {
@@ -31,23 +41,53 @@ __device__ __forceinline__ float ld_code(const void* p, int code, long i) {
   return code == 1 ? reinterpret_cast<const float*>(p)[i] : (float)reinterpret_cast<const bf16*>(p)[i];
 }
 
+// one block per token.  a [T, H*D] -> g in place; delta: aux[t] = [rq, rk per key/value head | b per head]
+template <typename TQ, bool DELTA>
+__global__ void scan_prep_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, long sk,
+                                 float* __restrict__ a, long sa, const float* __restrict__ a_bias,
+                                 const float* __restrict__ A_log, const void* __restrict__ beta, long sbeta,
+                                 int beta_code, float tau_inv, float* __restrict__ aux, int H, int G, int D) {
+  const long t = blockIdx.x;
+  float* ar = a + t * sa;
+  for (int e = threadIdx.x; e < H * D; e += blockDim.x) {
+    const float z = ar[e] + a_bias[e];
+    ar[e] = DELTA ? expf(-expf(A_log[e / D]) * mx_softplus(z)) : expf(-mx_softplus(-z) * tau_inv);
+  }
+  if (!DELTA) return;
+  float* ax = aux + t * (2 * G + H);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  const float qscale = 1.0f / sqrtf((float)D);
+  for (int r = wave; r < 2 * G; r += nw) {          // row r: q head r / 2 or k head r / 2
+    const TQ* src = (r & 1) ? k + t * sk + (r >> 1) * D : q + t * sq + (r >> 1) * D;
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) {
+      const float x = ldf(src + d);
+      ss += x * x;
+    }
+    ss = mx_wave_sum(ss);
+    if (lane == 0) ax[r] = ((r & 1) ? 1.0f : qscale) / sqrtf(ss + 1e-6f);
+  }
+  for (int h = threadIdx.x; h < H; h += blockDim.x) ax[2 * G + h] = mx_sigmoid(ld_code(beta, beta_code, t * sbeta + h));
+}
+
 // grid (ceil(P / CB), H, S), 256 threads = CB columns x LPC lanes, CB = 256 / LPC
-template <typename TQ, int RPL, int LPC, bool DELTA>
+template <typename TQ, int RPL, int LPC, bool DELTA, bool ONE>      // ONE: every segment is a single row (decode)
 __global__ void __launch_bounds__(256)
 matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, long sk, const TQ* __restrict__ v, long sv,
-                   const float* __restrict__ a, long sa, const float* __restrict__ a_bias,
-                   const float* __restrict__ A_log, const void* __restrict__ beta, long sbeta, int beta_code,
-                   float tau_inv, float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slot,
-                   const int* __restrict__ pos, float* __restrict__ out, int H, int G, int D, int P, int TB) {
-  extern __shared__ __align__(16) float lds[];
+                   const float* __restrict__ gdec, long sa, const float* __restrict__ aux, float* __restrict__ state,
+                   const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ pos,
+                   float* __restrict__ out, int H, int G, int D, int P) {
   constexpr int DP = RPL * LPC;          // padded key size
   constexpr int CB = 256 / LPC;          // columns per block
-  float* qs = lds;                       // [TB][DP]
-  float* ks = qs + TB * DP;              // [TB][DP]
-  float* gs = ks + TB * DP;              // [TB][DP]
-  float* vs = gs + TB * DP;              // [TB][CB]
-  float* os = vs + TB * CB;              // [TB][CB]
-  float* bs = os + TB * CB;              // [TB]
+  constexpr int TB = ONE ? 1 : (DP <= 256 ? 16 : 8);   // tokens per chunk
+  constexpr int NE = (TB * DP + 255) / 256;            // staged (token, key channel) elements per thread
+  constexpr int NV = (TB * CB + 255) / 256;
+  __shared__ __align__(16) float qs[TB * DP];
+  __shared__ __align__(16) float ks[TB * DP];
+  __shared__ __align__(16) float gs[TB * DP];
+  __shared__ float vs[TB * CB];
+  __shared__ float os[TB * CB];
+  __shared__ float bs[TB];
   const int s = blockIdx.z;
   const int sl = slot[s];
   if (sl < 0) return;
@@ -58,7 +98,7 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
   const int c0 = blockIdx.x * CB, col = c0 + cl;
   const bool fresh = pos[r0] == 0;
   const float qscale = 1.0f / sqrtf((float)D);
-  const float eA = DELTA ? expf(A_log[h]) : 0.f;
+  const int AW = 2 * G + H;              // aux row width
 
   float S[RPL];
   float* srec = state + (((long)sl * H + h) * D) * P;
@@ -68,46 +108,51 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
     S[i] = (!fresh && d < D && col < P) ? srec[(long)d * P + col] : 0.f;
   }
 
+  // chunk rows in flight: element e = tid + 256 * i is (token e / DP, channel e % DP); loads are clamped
+  // to the segment's last row and to channel D - 1, and masked when they land
+  float pq[NE], pk[NE], pg[NE], pv[NV], pb = 0.f;
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+      const int e = min(tid + 256 * i, TB * DP - 1);
+      const int t = e / DP, d = e - t * DP;
+      const long row = r0 + min(t0 + t, n - 1);
+      const int dc = min(d, D - 1);
+      float rq = DELTA ? aux[row * AW + 2 * kvh] : 1.f, rk = DELTA ? aux[row * AW + 2 * kvh + 1] : 1.f;
+      pq[i] = ldf(q + row * sq + kvh * D + dc) * rq;
+      pk[i] = ldf(k + row * sk + kvh * D + dc) * rk;
+      pg[i] = gdec[row * sa + h * D + dc];
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = min(tid + 256 * i, TB * CB - 1);
+      const int t = e / CB, c = e - t * CB;
+      pv[i] = ldf(v + (long)(r0 + min(t0 + t, n - 1)) * sv + h * P + min(c0 + c, P - 1));
+    }
+    if (DELTA && tid < TB) pb = aux[(long)(r0 + min(t0 + tid, n - 1)) * AW + 2 * G + h];
+  };
+  fetch(0);
   for (int t0 = 0; t0 < n; t0 += TB) {
     const int nt = min(TB, n - t0);
-    // ---- stage the chunk's rows
-    for (int e = tid; e < nt * DP; e += 256) {
-      const int t = e / DP, d = e - t * DP;
-      const long row = r0 + t0 + t;
-      float qv = 0.f, kv = 0.f, g = 1.f;
-      if (d < D) {
-        qv = ldf(q + row * sq + kvh * D + d);
-        kv = ldf(k + row * sk + kvh * D + d);
-        const float z = a[row * sa + h * D + d] + a_bias[h * D + d];
-        if (DELTA) g = expf(-eA * mx_softplus(z));
-        else {
-          g = expf(-mx_softplus(-z) * tau_inv);          // sigmoid(z)^(1/tau)
-          qv *= qscale;
-        }
+    __syncthreads();                     // the previous chunk's outputs have left os; its rows are consumed
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+      const int e = tid + 256 * i;
+      if (e < TB * DP) {
+        const bool live = (e % DP) < D;
+        qs[e] = live ? pq[i] : 0.f;
+        ks[e] = live ? pk[i] : 0.f;
+        gs[e] = live ? pg[i] : 1.f;
       }
-      qs[e] = qv;
-      ks[e] = kv;
-      gs[e] = g;
     }
-    for (int e = tid; e < nt * CB; e += 256) {
-      const int t = e / CB, c = e - t * CB;
-      vs[e] = c0 + c < P ? ldf(v + (long)(r0 + t0 + t) * sv + h * P + c0 + c) : 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = tid + 256 * i;
+      if (e < TB * CB) vs[e] = (c0 + e % CB) < P ? pv[i] : 0.f;
     }
-    if (DELTA)
-      for (int t = tid; t < nt; t += 256) bs[t] = mx_sigmoid(ld_code(beta, beta_code, (long)(r0 + t0 + t) * sbeta + h));
+    if (DELTA && tid < TB) bs[tid] = pb;
     __syncthreads();
-    if (DELTA) {      // q and k become unit vectors: one wave per row
-      const int wave = tid >> 6, lane = tid & 63;
-      for (int r = wave; r < 2 * nt; r += 4) {
-        float* buf = r < nt ? qs + r * DP : ks + (r - nt) * DP;
-        float ss = 0.f;
-        for (int d = lane; d < DP; d += 64) ss += buf[d] * buf[d];
-        ss = mx_wave_sum(ss);
-        const float sc = (r < nt ? qscale : 1.0f) / sqrtf(ss + 1e-6f);
-        for (int d = lane; d < DP; d += 64) buf[d] *= sc;
-      }
-      __syncthreads();
-    }
+    if (t0 + TB < n) fetch(t0 + TB);
     // ---- the recurrence
     for (int t = 0; t < nt; ++t) {
       const float4* kr = reinterpret_cast<const float4*>(ks + t * DP + part * RPL);
@@ -147,14 +192,13 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
         o += S[4 * i4] * qq.x + S[4 * i4 + 1] * qq.y + S[4 * i4 + 2] * qq.z + S[4 * i4 + 3] * qq.w;
       }
       o = lane_group_sum<LPC>(o);
-      if (part == 0) os[t * CB + cl] = o;
+      if (part == 0) os[t * CB + cl] = DELTA ? o : o * qscale;     // delta: the scale is part of q's norm factor
     }
     __syncthreads();
     for (int e = tid; e < nt * CB; e += 256) {
       const int t = e / CB, c = e - t * CB;
       if (c0 + c < P) out[(long)(r0 + t0 + t) * H * P + h * P + c0 + c] = os[e];
     }
-    // the next chunk's staging writes qs/ks/gs/vs/bs only; os is rewritten after the barrier that follows it
   }
 #pragma unroll
   for (int i = 0; i < RPL; ++i) {
@@ -167,98 +211,164 @@ __device__ __forceinline__ float gelu_tanh_f(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-// grid (ceil(R / 64), S), 64 threads: one lane per channel
+// elementwise over [T, R]: z[.., zr] <- a, z[.., zi] <- sqrt(1 - a^2) i u, out <- gelu_tanh(y + y_bias)
 template <typename TY, typename TO>
-__global__ void lru_scan_kernel(const float* __restrict__ u, const float* __restrict__ z, int bsz, long T,
-                                const float* __restrict__ r_bias, const float* __restrict__ i_bias,
-                                const float* __restrict__ lam, const TY* __restrict__ y, long sy,
-                                const float* __restrict__ y_bias, float* __restrict__ state, const int* __restrict__ cu,
-                                const int* __restrict__ slot, const int* __restrict__ pos, TO* __restrict__ out, int R) {
+__global__ void lru_gates_kernel(const float* __restrict__ u, float* __restrict__ z, int bsz, long T,
+                                 const float* __restrict__ r_bias, const float* __restrict__ i_bias,
+                                 const float* __restrict__ lam, const TY* __restrict__ y, long sy,
+                                 const float* __restrict__ y_bias, TO* __restrict__ out, int R) {
+  const long total = T * R;
+  for (long e = blockIdx.x * (long)blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
+    const long t = e / R;
+    const int c = (int)(e - t * R);
+    const int b = c / bsz, j = c - b * bsz;
+    float* zp = z + ((long)b * T + t) * 2 * bsz + j;
+    const float r = mx_sigmoid(zp[0] + r_bias[c]);
+    const float i = mx_sigmoid(zp[bsz] + i_bias[c]);
+    const float la = -8.0f * r * mx_softplus(lam[c]);             // log a
+    zp[0] = expf(la);
+    zp[bsz] = sqrtf(-expm1f(2.0f * la)) * i * u[e];               // 1 - a^2 without cancellation
+    stf(out + e, gelu_tanh_f(ldf(y + t * sy + c) + (y_bias != nullptr ? y_bias[c] : 0.f)));
+  }
+}
+
+constexpr int LRU_CL = 16;      // tokens per thread
+constexpr int LRU_NC = 4;       // thread chunks per block iteration (256 threads: 64 channels x 4)
+
+// grid (ceil(R / 64), S).  z holds a | input term (lru_gates_kernel), out holds the GeLU branch.
+template <typename TO>
+__global__ void __launch_bounds__(256)
+lru_scan_kernel(const float* __restrict__ z, int bsz, long T, float* __restrict__ state, const int* __restrict__ cu,
+                const int* __restrict__ slot, const int* __restrict__ pos, TO* __restrict__ out, int R) {
+  __shared__ float sA[LRU_NC][64], sB[LRU_NC][64], sS[64];
   const int s = blockIdx.y;
   const int sl = slot[s];
   if (sl < 0) return;
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= R) return;
-  const int r0 = cu[s], r1 = cu[s + 1];
-  if (r1 <= r0) return;
-  const int b = c / bsz, j = c - b * bsz;
-  const float* zb = z + (long)b * T * 2 * bsz + j;     // block b's rows: [T][zr: bsz | zi: bsz]
-  const float sp = mx_softplus(lam[c]), rb = r_bias[c], ib = i_bias[c];
-  const float yb = y_bias != nullptr ? y_bias[c] : 0.f;
-  float S = pos[r0] == 0 ? 0.f : state[(long)sl * R + c];
-#pragma unroll 4
-  for (long t = r0; t < r1; ++t) {
-    const float r = mx_sigmoid(zb[t * 2 * bsz] + rb);
-    const float i = mx_sigmoid(zb[t * 2 * bsz + bsz] + ib);
-    const float la = -8.0f * r * sp;                   // log a
-    S = expf(la) * S + sqrtf(-expm1f(2.0f * la)) * i * u[t * R + c];
-    stf(out + t * R + c, S * gelu_tanh_f(ldf(y + t * sy + c) + yb));
+  const int r0 = cu[s], n = cu[s + 1] - r0;
+  if (n <= 0) return;
+  const int ch = threadIdx.x & 63, j = threadIdx.x >> 6;
+  const int c = min((int)blockIdx.x * 64 + ch, R - 1);
+  const bool live = (int)blockIdx.x * 64 + ch < R;
+  const int b = c / bsz, jj = c - b * bsz;
+  const float* zb = z + (long)b * T * 2 * bsz + jj;
+  if (j == 0) sS[ch] = pos[r0] == 0 ? 0.f : state[(long)sl * R + c];
+  for (int t0 = 0; t0 < n; t0 += LRU_CL * LRU_NC) {
+    const int first = t0 + j * LRU_CL;
+    const int cnt = max(0, min(LRU_CL, n - first));
+    float A[LRU_CL], L[LRU_CL], Gy[LRU_CL];
+#pragma unroll
+    for (int i = 0; i < LRU_CL; ++i) {          // independent loads, issued together
+      const long t = r0 + min(first + i, n - 1);
+      A[i] = zb[t * 2 * bsz];
+      L[i] = zb[t * 2 * bsz + bsz];
+      Gy[i] = ldf(out + t * R + c);
+    }
+    float Pp = 1.f, Ll = 0.f;
+#pragma unroll
+    for (int i = 0; i < LRU_CL; ++i) {
+      if (i < cnt) {
+        Ll = A[i] * Ll + L[i];
+        Pp *= A[i];
+      }
+      L[i] = Ll;      // state after token i from a zero start
+      A[i] = Pp;      // product of the decays up to token i
+    }
+    sA[j][ch] = Pp;
+    sB[j][ch] = Ll;
+    __syncthreads();
+    float S0 = sS[ch];
+    for (int k = 0; k < j; ++k) S0 = sA[k][ch] * S0 + sB[k][ch];
+#pragma unroll
+    for (int i = 0; i < LRU_CL; ++i)
+      if (i < cnt && live) stf(out + (long)(r0 + first + i) * R + c, (L[i] + A[i] * S0) * Gy[i]);
+    __syncthreads();                             // every thread has read sS and the partial maps
+    if (j == LRU_NC - 1) sS[ch] = Pp * S0 + Ll;
+    __syncthreads();
   }
-  state[(long)sl * R + c] = S;
+  if (j == 0 && live) state[(long)sl * R + c] = sS[ch];
 }
 
 template <typename TQ, int RPL, int LPC, bool DELTA>
-int launch_matrix_scan(const void* q, long sq, const void* k, long sk, const void* v, long sv, const float* a, long sa,
-                       const float* a_bias, const float* A_log, const void* beta, long sbeta, int beta_code,
-                       float tau_inv, float* state, const int* cu, const int* slot, const int* pos, float* out, int S,
-                       int H, int G, int D, int P, hipStream_t st) {
-  constexpr int DP = RPL * LPC, CB = 256 / LPC;
-  const int per_tok = (3 * DP + 2 * CB + 1) * (int)sizeof(float);
-  int TB = (44 * 1024) / per_tok;
-  TB = TB > 16 ? 16 : (TB < 1 ? 1 : TB);
+int launch_matrix_scan(const void* q, long sq, const void* k, long sk, const void* v, long sv, const float* g, long sa,
+                       const float* aux, float* state, const int* cu, const int* slot, const int* pos, float* out, int S,
+                       int H, int G, int D, int P, bool one, hipStream_t st) {
+  constexpr int CB = 256 / LPC;
   dim3 grid((P + CB - 1) / CB, H, S);
-  matrix_scan_kernel<TQ, RPL, LPC, DELTA><<<grid, 256, (size_t)TB * per_tok, st>>>(
-      (const TQ*)q, sq, (const TQ*)k, sk, (const TQ*)v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_code, tau_inv, state,
-      cu, slot, pos, out, H, G, D, P, TB);
+  if (one)
+    matrix_scan_kernel<TQ, RPL, LPC, DELTA, true><<<grid, 256, 0, st>>>(
+        (const TQ*)q, sq, (const TQ*)k, sk, (const TQ*)v, sv, g, sa, aux, state, cu, slot, pos, out, H, G, D, P);
+  else
+    matrix_scan_kernel<TQ, RPL, LPC, DELTA, false><<<grid, 256, 0, st>>>(
+        (const TQ*)q, sq, (const TQ*)k, sk, (const TQ*)v, sv, g, sa, aux, state, cu, slot, pos, out, H, G, D, P);
   MX_RETURN_LAUNCH();
 }
 
+// the variant with 16 lanes per column when the narrow one would leave most of the chip idle
 template <typename TQ, bool DELTA, typename... Args>
-int dispatch_matrix_scan(int D, Args... args) {
+int dispatch_matrix_scan(int D, bool wide, Args... args) {
   if (D <= 32) return launch_matrix_scan<TQ, 8, 4, DELTA>(args...);
-  if (D <= 64) return launch_matrix_scan<TQ, 16, 4, DELTA>(args...);
-  if (D <= 128) return launch_matrix_scan<TQ, 32, 4, DELTA>(args...);
-  if (D <= 256) return launch_matrix_scan<TQ, 32, 8, DELTA>(args...);
+  if (D <= 64) return wide ? launch_matrix_scan<TQ, 4, 16, DELTA>(args...) : launch_matrix_scan<TQ, 16, 4, DELTA>(args...);
+  if (D <= 128) return wide ? launch_matrix_scan<TQ, 8, 16, DELTA>(args...) : launch_matrix_scan<TQ, 32, 4, DELTA>(args...);
+  if (D <= 256) return wide ? launch_matrix_scan<TQ, 16, 16, DELTA>(args...) : launch_matrix_scan<TQ, 32, 8, DELTA>(args...);
   return launch_matrix_scan<TQ, 32, 16, DELTA>(args...);
+}
+
+template <typename TQ, bool DELTA>
+int run_matrix_scan(const void* q, long sq, const void* k, long sk, const void* v, long sv, float* a, long sa,
+                    const float* a_bias, const float* A_log, const void* beta, long sbeta, int beta_dt, float tau_inv,
+                    float* aux, float* state, const int* cu, const int* slot, const int* pos, float* out, int S, int T,
+                    int H, int G, int D, int P, bool one, hipStream_t st) {
+  scan_prep_kernel<TQ, DELTA><<<T, 256, 0, st>>>((const TQ*)q, sq, (const TQ*)k, sk, a, sa, a_bias, A_log, beta, sbeta,
+                                                 beta_dt, tau_inv, aux, H, G, D);
+  const int lpc = D <= 128 ? 4 : (D <= 256 ? 8 : 16);
+  const long blocks = (long)S * H * ((P + 256 / lpc - 1) / (256 / lpc));
+  return dispatch_matrix_scan<TQ, DELTA>(D, blocks < 512, q, sq, k, sk, v, sv, (const float*)a, sa, (const float*)aux, state,
+                                         cu, slot, pos, out, S, H, G, D, P, one, st);
 }
 
 }  // namespace
 
-// q, k [rows, G*D] and v [rows, H*P] slices of storage type dt (row strides sq, sk, sv); a f32 [rows, H*D]
-// slice (row stride sa); a_bias f32 [H*D]; delta != 0: A_log f32 [H], beta [rows, >= H] slice of type
-// beta_dt; state f32 [slots, H, D, P]; out f32 [rows, H*P].
-MX_API int mx_matrix_scan(const void* q, long sq, const void* k, long sk, const void* v, long sv, int dt, const float* a,
+// q, k [rows, G*D] and v [rows, H*P] slices of storage type dt (row strides sq, sk, sv); a f32 [T, H*D]
+// slice (row stride sa), OVERWRITTEN with the decays; a_bias f32 [H*D]; delta != 0: A_log f32 [H], beta
+// [T, >= H] slice of type beta_dt, aux f32 [T, 2*G + H] scratch; state f32 [slots, H, D, P]; out f32
+// [T, H*P].  T: rows of the step (every row belongs to a segment or is padding); max_len: the longest
+// segment (1: the decode form).
+MX_API int mx_matrix_scan(const void* q, long sq, const void* k, long sk, const void* v, long sv, int dt, float* a,
                           long sa, const float* a_bias, const float* A_log, const void* beta, long sbeta, int beta_dt,
-                          float tau, int delta, float* state, const int* cu, const int* slot, const int* pos,
-                          float* out, int S, int H, int G, int D, int P, hipStream_t st) {
-  if (S <= 0) return 0;
-  if (D < 1 || D > 512 || G < 1 || H % G || (delta && (A_log == nullptr || beta == nullptr)) || tau <= 0.f)
+                          float tau, int delta, float* aux, float* state, const int* cu, const int* slot, const int* pos,
+                          float* out, int S, int T, int max_len, int H, int G, int D, int P, hipStream_t st) {
+  if (S <= 0 || T <= 0) return 0;
+  const bool one = max_len == 1;         // every segment is a single row: no chunk staging
+  if (D < 1 || D > 512 || G < 1 || H % G || tau <= 0.f || (delta && (A_log == nullptr || beta == nullptr || aux == nullptr)))
     return (int)hipErrorInvalidValue;
-  const float tau_inv = 1.0f / tau;
+  const float ti = 1.0f / tau;
   if (delta) {
     if (dt == 1)
-      return dispatch_matrix_scan<float, true>(D, q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt,
-                                               tau_inv, state, cu, slot, pos, out, S, H, G, D, P, st);
-    return dispatch_matrix_scan<bf16, true>(D, q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, tau_inv,
-                                            state, cu, slot, pos, out, S, H, G, D, P, st);
+      return run_matrix_scan<float, true>(q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, ti, aux, state,
+                                          cu, slot, pos, out, S, T, H, G, D, P, one, st);
+    return run_matrix_scan<bf16, true>(q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, ti, aux, state, cu,
+                                       slot, pos, out, S, T, H, G, D, P, one, st);
   }
   if (dt == 1)
-    return dispatch_matrix_scan<float, false>(D, q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt,
-                                              tau_inv, state, cu, slot, pos, out, S, H, G, D, P, st);
-  return dispatch_matrix_scan<bf16, false>(D, q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, tau_inv,
-                                           state, cu, slot, pos, out, S, H, G, D, P, st);
+    return run_matrix_scan<float, false>(q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, ti, aux, state,
+                                         cu, slot, pos, out, S, T, H, G, D, P, one, st);
+  return run_matrix_scan<bf16, false>(q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, ti, aux, state, cu,
+                                      slot, pos, out, S, T, H, G, D, P, one, st);
 }
 
-// u f32 [T, R]; z f32 [blocks, T, 2 * R / blocks]; y [T, >= R] slice (row stride sy, type dt_y); state f32
-// [slots, R]; out [T, R] of type dt_out
-MX_API int mx_lru_scan(const float* u, const float* z, int blocks, const float* r_bias, const float* i_bias,
+// u f32 [T, R]; z f32 [blocks, T, 2 * R / blocks], OVERWRITTEN with the gates; y [T, >= R] slice (row stride
+// sy, type dt_y); state f32 [slots, R]; out [T, R] of type dt_out
+MX_API int mx_lru_scan(const float* u, float* z, int blocks, const float* r_bias, const float* i_bias,
                        const float* lam, const void* y, long sy, int dt_y, const float* y_bias, float* state,
                        const int* cu, const int* slot, const int* pos, void* out, int dt_out, int S, int R, int T,
                        hipStream_t st) {
   if (S <= 0 || T <= 0) return 0;
   if (blocks < 1 || R % blocks) return (int)hipErrorInvalidValue;
+  const long total = (long)T * R;
+  const int gb = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+  MX_DISPATCH(dt_y, TY, MX_DISPATCH(dt_out, TO, lru_gates_kernel<TY, TO><<<gb, 256, 0, st>>>(
+      u, z, R / blocks, (long)T, r_bias, i_bias, lam, (const TY*)y, sy, y_bias, (TO*)out, R)));
   dim3 grid((R + 63) / 64, S);
-  MX_DISPATCH(dt_y, TY, MX_DISPATCH(dt_out, TO, lru_scan_kernel<TY, TO><<<grid, 64, 0, st>>>(
-      u, z, R / blocks, (long)T, r_bias, i_bias, lam, (const TY*)y, sy, y_bias, state, cu, slot, pos, (TO*)out, R)));
+  MX_DISPATCH(dt_out, TO, lru_scan_kernel<TO><<<grid, 256, 0, st>>>(z, R / blocks, (long)T, state, cu, slot, pos, (TO*)out, R));
   MX_RETURN_LAUNCH();
 }

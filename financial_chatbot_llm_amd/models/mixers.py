@@ -385,7 +385,8 @@ class ChannelDeltaMixer:
         beta = proj[:, C:C + H]
         a = F.linear(proj[:, C + H:C + H + self.ra].float(), self.a2)
         o = mx.matrix_scan(u[:, :nq], u[:, nq:2 * nq], u[:, 2 * nq:], a, self.dt_bias, st["S"], meta.seg_cu,
-                           meta.seg_state, positions, H, self.G, self.D, self.P, "delta", A_log=self.A_log, beta=beta)
+                           meta.seg_state, positions, H, self.G, self.D, self.P, "delta", A_log=self.A_log, beta=beta,
+                           max_len=meta.seg_max_len)
         gate = F.linear(proj[:, C + H + self.ra:C + H + self.ra + self.rg], self.g2)
         return F.linear(mx.head_norm_gate(o, self.norm_w, self.eps, gate, H, "sigmoid", proj.dtype), self.o)
 
@@ -429,7 +430,8 @@ class GLAMixer:
         nq, nv = self.nq, self.nv
         a = F.linear(proj[:, 2 * nq + 2 * nv:2 * nq + 2 * nv + self.ra].float(), self.a2)
         o = mx.matrix_scan(proj[:, :nq], proj[:, nq:2 * nq], proj[:, 2 * nq:2 * nq + nv], a, self.a2_b, st["S"],
-                           meta.seg_cu, meta.seg_state, positions, self.H, self.H, self.D, self.P, "gla", tau=self.tau)
+                           meta.seg_cu, meta.seg_state, positions, self.H, self.H, self.D, self.P, "gla", tau=self.tau,
+                           max_len=meta.seg_max_len)
         gate = proj[:, 2 * nq + nv:2 * nq + 2 * nv]
         return F.linear(mx.head_norm_gate(o, self.norm_w, self.eps, gate, self.H, "silu", proj.dtype), self.o)
 

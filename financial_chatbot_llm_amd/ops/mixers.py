@@ -511,17 +511,18 @@ def conv_act(inp: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], s
 def matrix_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tensor, a_bias: torch.Tensor,
                 state: torch.Tensor, cu: torch.Tensor, slot: torch.Tensor, pos: torch.Tensor, heads: int, kv_heads: int,
                 dim: int, vdim: int, mode: str, tau: float = 1.0, A_log: Optional[torch.Tensor] = None,
-                beta: Optional[torch.Tensor] = None) -> torch.Tensor:
+                beta: Optional[torch.Tensor] = None, max_len: int = 0) -> torch.Tensor:
     """Token-by-token f32 recurrence over a [dim, vdim] state per head (``state`` f32
     [slots, H, dim, vdim], read unless the segment starts at position 0, then replaced), with one
     decay per head and key channel acting on the state's rows.  ``q``/``k`` [T, G*dim], ``v``
     [T, H*vdim] (column slices; head h reads q/k head h // (H/G)), ``a`` f32 [T, H*dim] the decay's
-    pre-activation, ``a_bias`` f32 [H*dim].
+    pre-activation (the kernels overwrite it with the decays), ``a_bias`` f32 [H*dim].
 
     ``mode="gla"``:   g = sigmoid(a + a_bias)^(1/tau);  S <- g S + k v^T;  o = S^T (q dim^-1/2).
     ``mode="delta"``: q, k <- unit vectors (x / sqrt(sum x^2 + 1e-6)), q scaled by dim^-1/2;
                       g = exp(-exp(A_log[h]) softplus(a + a_bias));  b = sigmoid(beta[t, h]);
                       S <- g S;  u = b (v - S^T k);  S <- S + k u^T;  o = S^T q.
+    ``max_len``: the longest segment when known (1 selects the kernels' single-row form).
     Returns o f32 [T, H*vdim]."""
     T = q.shape[0]
     H, G, D, P = heads, kv_heads, dim, vdim
@@ -531,11 +532,12 @@ def matrix_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tens
     assert q.dtype == k.dtype == v.dtype
     if N.use_native(q):
         out = torch.empty((T, H * P), dtype=torch.float32, device=q.device)
+        aux = torch.empty((T, 2 * G + H), dtype=torch.float32, device=q.device) if delta else None
         N.mcall("mx_matrix_scan", N.ptr(_rows(q)), q.stride(0), N.ptr(_rows(k)), k.stride(0), N.ptr(_rows(v)), v.stride(0),
                 _dt(q), N.ptr(_rows(a)), a.stride(0), N.ptr(a_bias), N.ptr(A_log) if delta else None,
                 N.ptr(_rows(beta)) if delta else None, beta.stride(0) if delta else 0, _dt(beta) if delta else 1,
-                float(tau), 1 if delta else 0, N.ptr(state), N.ptr(cu), N.ptr(slot), N.ptr(pos), N.ptr(out), S, H, G, D, P,
-                N.stream())
+                float(tau), 1 if delta else 0, N.ptr(aux), N.ptr(state), N.ptr(cu), N.ptr(slot), N.ptr(pos), N.ptr(out), S, T,
+                int(max_len), H, G, D, P, N.stream())
         return out
     out = torch.zeros((T, H * P), dtype=torch.float32)
     cul, sll, pl = cu.tolist(), slot.tolist(), pos.tolist()
@@ -595,7 +597,8 @@ def lru_scan(u: torch.Tensor, z: torch.Tensor, blocks: int, r_bias: torch.Tensor
     """Per channel, f32: r = sigmoid(zr + r_bias), i = sigmoid(zi + i_bias), a = exp(-8 r softplus(lam)),
     S <- a S + sqrt(1 - a^2) i u (also for a sequence's first token, from S = 0); returns
     S * gelu_tanh(y + y_bias) in ``out_dtype``.  ``u`` f32 [T, R]; ``z`` f32 [blocks, T, 2 * R / blocks]:
-    block b's gate pre-activations [zr | zi] as the batched block-diagonal product leaves them;
+    block b's gate pre-activations [zr | zi] as the batched block-diagonal product leaves them (the
+    kernels overwrite it with the gates);
     ``y`` a column slice; ``state`` f32 [slots, R], read unless the segment starts at position 0,
     then replaced."""
     T, R = u.shape
