@@ -7,7 +7,8 @@
 //             S <- S + k u^T;  o = S^T q;    q, k unit vectors per head first, b = sigmoid(beta)
 //   and q scaled by D^-1/2 in both.  Two launches:
 //     prep   one block per token, fully parallel: the decays g (written over `a`), and for the delta
-//            rule the unit-norm factors of q and k and sigmoid(beta);
+//            rule the unit-norm factors of q and k and sigmoid(beta) (steps of single rows -- decode --
+//            skip this launch: the scan's one-token form computes them while it stages the row);
 //     scan   column p of S never meets another column, so a lane owns RPL rows of one column in
 //            registers and LPC neighbouring lanes share a column (D <= RPL * LPC); the two dot
 //            products per token are reduced over those lanes with DPP swaps.  The rows of a chunk
@@ -76,7 +77,9 @@ __global__ void __launch_bounds__(256)
 matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, long sk, const TQ* __restrict__ v, long sv,
                    const float* __restrict__ gdec, long sa, const float* __restrict__ aux, float* __restrict__ state,
                    const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ pos,
-                   float* __restrict__ out, int H, int G, int D, int P) {
+                   float* __restrict__ out, int H, int G, int D, int P, const float* __restrict__ a_bias,
+                   const float* __restrict__ A_log, const void* __restrict__ beta, long sbeta, int beta_code,
+                   float tau_inv) {
   constexpr int DP = RPL * LPC;          // padded key size
   constexpr int CB = 256 / LPC;          // columns per block
   constexpr int TB = ONE ? 1 : (DP <= 256 ? 16 : 8);   // tokens per chunk
@@ -118,10 +121,17 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
       const int t = e / DP, d = e - t * DP;
       const long row = r0 + min(t0 + t, n - 1);
       const int dc = min(d, D - 1);
-      float rq = DELTA ? aux[row * AW + 2 * kvh] : 1.f, rk = DELTA ? aux[row * AW + 2 * kvh + 1] : 1.f;
-      pq[i] = ldf(q + row * sq + kvh * D + dc) * rq;
-      pk[i] = ldf(k + row * sk + kvh * D + dc) * rk;
-      pg[i] = gdec[row * sa + h * D + dc];
+      if (ONE) {       // no prep pass ran: the decay from its pre-activation here, the unit norms after staging
+        pq[i] = ldf(q + row * sq + kvh * D + dc);
+        pk[i] = ldf(k + row * sk + kvh * D + dc);
+        const float z = gdec[row * sa + h * D + dc] + a_bias[h * D + dc];
+        pg[i] = DELTA ? expf(-expf(A_log[h]) * mx_softplus(z)) : expf(-mx_softplus(-z) * tau_inv);
+      } else {
+        float rq = DELTA ? aux[row * AW + 2 * kvh] : 1.f, rk = DELTA ? aux[row * AW + 2 * kvh + 1] : 1.f;
+        pq[i] = ldf(q + row * sq + kvh * D + dc) * rq;
+        pk[i] = ldf(k + row * sk + kvh * D + dc) * rk;
+        pg[i] = gdec[row * sa + h * D + dc];
+      }
     }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -129,7 +139,9 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
       const int t = e / CB, c = e - t * CB;
       pv[i] = ldf(v + (long)(r0 + min(t0 + t, n - 1)) * sv + h * P + min(c0 + c, P - 1));
     }
-    if (DELTA && tid < TB) pb = aux[(long)(r0 + min(t0 + tid, n - 1)) * AW + 2 * G + h];
+    if (DELTA && tid < TB)
+      pb = ONE ? mx_sigmoid(ld_code(beta, beta_code, (long)(r0 + min(t0 + tid, n - 1)) * sbeta + h))
+               : aux[(long)(r0 + min(t0 + tid, n - 1)) * AW + 2 * G + h];
   };
   fetch(0);
   for (int t0 = 0; t0 < n; t0 += TB) {
@@ -152,6 +164,18 @@ matrix_scan_kernel(const TQ* __restrict__ q, long sq, const TQ* __restrict__ k, 
     }
     if (DELTA && tid < TB) bs[tid] = pb;
     __syncthreads();
+    if (ONE && DELTA) {                  // q (wave 0) and k (wave 1) become unit vectors
+      const int wave = tid >> 6, lane = tid & 63;
+      if (wave < 2) {
+        float* buf = wave == 0 ? qs : ks;
+        float ss = 0.f;
+        for (int d = lane; d < DP; d += 64) ss += buf[d] * buf[d];
+        ss = mx_wave_sum(ss);
+        const float sc = (wave == 0 ? qscale : 1.0f) / sqrtf(ss + 1e-6f);
+        for (int d = lane; d < DP; d += 64) buf[d] *= sc;
+      }
+      __syncthreads();
+    }
     if (t0 + TB < n) fetch(t0 + TB);
     // ---- the recurrence
     for (int t = 0; t < nt; ++t) {
@@ -291,15 +315,18 @@ lru_scan_kernel(const float* __restrict__ z, int bsz, long T, float* __restrict_
 template <typename TQ, int RPL, int LPC, bool DELTA>
 int launch_matrix_scan(const void* q, long sq, const void* k, long sk, const void* v, long sv, const float* g, long sa,
                        const float* aux, float* state, const int* cu, const int* slot, const int* pos, float* out, int S,
-                       int H, int G, int D, int P, bool one, hipStream_t st) {
+                       int H, int G, int D, int P, const float* a_bias, const float* A_log, const void* beta, long sbeta,
+                       int beta_dt, float tau_inv, bool one, hipStream_t st) {
   constexpr int CB = 256 / LPC;
   dim3 grid((P + CB - 1) / CB, H, S);
   if (one)
     matrix_scan_kernel<TQ, RPL, LPC, DELTA, true><<<grid, 256, 0, st>>>(
-        (const TQ*)q, sq, (const TQ*)k, sk, (const TQ*)v, sv, g, sa, aux, state, cu, slot, pos, out, H, G, D, P);
+        (const TQ*)q, sq, (const TQ*)k, sk, (const TQ*)v, sv, g, sa, aux, state, cu, slot, pos, out, H, G, D, P, a_bias,
+        A_log, beta, sbeta, beta_dt, tau_inv);
   else
     matrix_scan_kernel<TQ, RPL, LPC, DELTA, false><<<grid, 256, 0, st>>>(
-        (const TQ*)q, sq, (const TQ*)k, sk, (const TQ*)v, sv, g, sa, aux, state, cu, slot, pos, out, H, G, D, P);
+        (const TQ*)q, sq, (const TQ*)k, sk, (const TQ*)v, sv, g, sa, aux, state, cu, slot, pos, out, H, G, D, P, a_bias,
+        A_log, beta, sbeta, beta_dt, tau_inv);
   MX_RETURN_LAUNCH();
 }
 
@@ -318,12 +345,14 @@ int run_matrix_scan(const void* q, long sq, const void* k, long sk, const void* 
                     const float* a_bias, const float* A_log, const void* beta, long sbeta, int beta_dt, float tau_inv,
                     float* aux, float* state, const int* cu, const int* slot, const int* pos, float* out, int S, int T,
                     int H, int G, int D, int P, bool one, hipStream_t st) {
-  scan_prep_kernel<TQ, DELTA><<<T, 256, 0, st>>>((const TQ*)q, sq, (const TQ*)k, sk, a, sa, a_bias, A_log, beta, sbeta,
-                                                 beta_dt, tau_inv, aux, H, G, D);
+  if (!one)        // single-row steps fold this pass into the scan (one launch less per layer)
+    scan_prep_kernel<TQ, DELTA><<<T, 256, 0, st>>>((const TQ*)q, sq, (const TQ*)k, sk, a, sa, a_bias, A_log, beta, sbeta,
+                                                   beta_dt, tau_inv, aux, H, G, D);
   const int lpc = D <= 128 ? 4 : (D <= 256 ? 8 : 16);
   const long blocks = (long)S * H * ((P + 256 / lpc - 1) / (256 / lpc));
   return dispatch_matrix_scan<TQ, DELTA>(D, blocks < 512, q, sq, k, sk, v, sv, (const float*)a, sa, (const float*)aux, state,
-                                         cu, slot, pos, out, S, H, G, D, P, one, st);
+                                         cu, slot, pos, out, S, H, G, D, P, a_bias, A_log, beta, sbeta, beta_dt, tau_inv,
+                                         one, st);
 }
 
 }  // namespace
