@@ -5,7 +5,7 @@
   it with ctypes (``ops/_native.py``); no torch headers are involved, so a full rebuild takes
   seconds and the library loads into the same HIP runtime torch already initialised.
 * ``libpenny_mixers.so`` -- ``csrc/mixers/*.hip``: the sequence-mixer kernels of the hybrid decoders
-  (state-space scan, latent attention, biased routing, the 32-bit residual stream), a library of
+  (state-space and matrix-state scans, latent and windowed attention, routing, the 32-bit residual stream), a library of
   its own so that a model that needs only these compiles only these (``build_mixers``).
 * ``libpenny_kernels_debug.so`` (``--debug``) -- the same kernels with device-side bounds checks
   (``PENNY_DASSERT`` in ``common.h``), loaded instead when ``PENNY_KERNEL_DEBUG=1``.

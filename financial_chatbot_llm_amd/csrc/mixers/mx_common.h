@@ -1,5 +1,5 @@
-// Shared helpers of the sequence-mixer kernel library (gfx950): state-space scans, latent
-// attention, biased top-k routing and the 32-bit residual stream of the hybrid decoders.
+// Shared helpers of the sequence-mixer kernel library (gfx950): state-space and matrix-state scans,
+// latent and windowed attention, top-k routing and the 32-bit residual stream of the layered decoders.
 //
 // Conventions: wave = 64 lanes; every launcher is `extern "C"`, takes raw device pointers and a
 // hipStream_t, never allocates or synchronises (hipGraph-capturable) and returns the launch's

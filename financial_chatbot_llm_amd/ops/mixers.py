@@ -1,7 +1,11 @@
 """Sequence-mixer ops of the hybrid decoders (``csrc/mixers``): a 32-bit residual stream with a fused
 parallel-block update + RMS norm, grouped / gated RMS norms, the Mamba-2 causal convolution and
 state-space scan over a flat batch of segments, latent attention over a paged latent cache with a
-sliding window, clamped gated units, and biased top-k routing.
+sliding window, clamped gated units, and biased top-k routing; and, for the sequential post-norm
+decoders, a hashed token-pair embedding, layer norm on the sublayer output fused with the residual
+add, matrix-state linear recurrences (gated linear attention, gated delta rule), a real-gated linear
+recurrent unit, sliding-window attention with grouped key/value heads over a paged [k | v] row cache,
+gated activations with a per-row scale and sigmoid top-k routing.
 
 Activations are bf16 or f32 (a model-wide choice); statistics, scores, softmax, recurrences and the
 residual stream are f32 either way.  CUDA(HIP) tensors run the kernels of ``libpenny_mixers.so``
