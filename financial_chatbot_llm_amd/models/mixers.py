@@ -185,7 +185,7 @@ class DenseFF:
     def num_bytes(self) -> int:
         return self.down.numel() * self.down.element_size()
 
-    def forward(self, h: torch.Tensor, proj: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, proj: torch.Tensor, x32: Optional[torch.Tensor] = None) -> torch.Tensor:
         if self.gated:
             return F.linear(mx.glu_act(proj[:, :self.ff], proj[:, self.ff:2 * self.ff], self.act), self.down)
         return F.linear(mx.relu2(proj), self.down)
@@ -298,10 +298,12 @@ class InputScaledRoutedFF:
     def num_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.router, self.w13, self.w2))
 
-    def forward(self, h: torch.Tensor, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, proj: Optional[torch.Tensor] = None, x32: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``x32``: the f32 input ``h`` was rounded from, when the caller has it: the router then reads the
+        unrounded values (fewer swapped near-ties against an exact evaluation)."""
         T, W = h.shape
         E, top, Fe = self.E, self.top, self.F
-        wts, idx = mx.route_scores(F.linear(h.float(), self.router), top, self.score)
+        wts, idx = mx.route_scores(F.linear(x32 if x32 is not None else h.float(), self.router), top, self.score)
         ones = torch.ones_like(wts)
         if T * top <= DENSE_MAX_PAIRS or _capturing(h):
             # every expert over every row; rows an expert was not chosen for get scale 0 and are not read

@@ -135,7 +135,7 @@ class SigudraModel(LayeredDecoder):
             else:
                 h = mx.post_norm_add(x, m, l.norm1, eps, dt)
             if l.ff is not None:
-                f = l.ff.forward(h, F.linear(h, l.w_ff) if l.w_ff is not None else None)
+                f = l.ff.forward(h, F.linear(h, l.w_ff) if l.w_ff is not None else None, x32=x)
                 h = mx.post_norm_add(x, f, l.norm2, eps, dt)
             if self.capture is not None:
                 self.capture.append(x.clone())
