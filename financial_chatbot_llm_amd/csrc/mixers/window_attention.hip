@@ -185,7 +185,8 @@ window_attend_kernel(const T* __restrict__ q, long sq, const T* __restrict__ cac
 //     S^T = K . Q^T      A: key rows from LDS (16-byte reads), B: the wave's queries, in registers
 //     online softmax     the statistics of query (lane % 16) live in that lane, f32
 //     O^T += V^T . P^T   A: the value tile, transposed in LDS; B: P straight from the S^T registers
-//                        (the MFMA's k slots 8g+i / 8g+4+i hold keys 4g+i / 16+4g+i)
+//                        (the MFMA's k slots 8g+i / 8g+4+i hold keys 4g+i / 16+4g+i), as two bf16
+//                        terms hi + lo so that the f32 softmax weights are not cut to 8 bits
 // Feature dimensions are zero-padded to multiples of 32 (keys) / 16 (values) in LDS and registers.
 // Single-row segments (decode) may split each row's key range over nsplit blocks; the parts
 // (unnormalised output, running maximum, sum) are combined by window_merge_kernel.
@@ -350,7 +351,9 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float mn = fmaxf(m, tmax);
     const float corr = (m == -INFINITY) ? 0.f : expf(m - mn);
-    bf16x8 pb;
+    // the f32 weight enters the value product as two bf16 terms, p = hi + lo (16 mantissa bits: far
+    // below the rounding of the bf16 values it multiplies), both accumulated in f32
+    bf16x8 pb, pl;
     float psum = 0.f;
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh)
@@ -358,7 +361,9 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
       for (int i = 0; i < 4; ++i) {
         const float p = sc[kh][i] == -INFINITY ? 0.f : expf(sc[kh][i] - mn);
         psum += p;
-        pb[4 * kh + i] = (bf16)p;
+        const bf16 hi = (bf16)p;
+        pb[4 * kh + i] = hi;
+        pl[4 * kh + i] = (bf16)(p - (float)hi);
       }
     psum += __shfl_xor(psum, 16, 64);
     psum += __shfl_xor(psum, 32, 64);
@@ -377,6 +382,7 @@ window_attend_mfma_kernel(const bf16* __restrict__ q, long sq, const bf16* __res
         }
         o[nt] *= corr;
         o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[nt], 0, 0, 0);
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pl, o[nt], 0, 0, 0);
       }
     }
   }
