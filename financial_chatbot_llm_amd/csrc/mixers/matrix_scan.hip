@@ -21,7 +21,7 @@
 // mx_lru_scan: a diagonal recurrence per channel, S <- a S + sqrt(1 - a^2) i u with
 //     a = exp(-8 sigmoid(zr + r_bias) softplus(lam)),  i = sigmoid(zi + i_bias),
 //   output S * gelu_tanh(y + y_bias).  Two launches: the gates (a, the input term and the GeLU
-//   branch: every transcendental) elementwise over all rows, then the recurrence itself, where a
+//   branch: every transcendental; they replace z and u in place, in f32) elementwise over all rows, then the recurrence itself, where a
 //   block walks 64 tokens at a time: each thread scans 16 tokens of one channel from zero, the four
 //   partial maps S -> A S + B are folded through LDS, and the outputs are corrected by the true
 //   start state.
@@ -235,12 +235,13 @@ __device__ __forceinline__ float gelu_tanh_f(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-// elementwise over [T, R]: z[.., zr] <- a, z[.., zi] <- sqrt(1 - a^2) i u, out <- gelu_tanh(y + y_bias)
-template <typename TY, typename TO>
-__global__ void lru_gates_kernel(const float* __restrict__ u, float* __restrict__ z, int bsz, long T,
+// elementwise over [T, R]: z[.., zr] <- a, z[.., zi] <- sqrt(1 - a^2) i u, then u <- gelu_tanh(y + y_bias)
+// (f32: the branch is rounded once, with the product, not before it)
+template <typename TY>
+__global__ void lru_gates_kernel(float* __restrict__ u, float* __restrict__ z, int bsz, long T,
                                  const float* __restrict__ r_bias, const float* __restrict__ i_bias,
                                  const float* __restrict__ lam, const TY* __restrict__ y, long sy,
-                                 const float* __restrict__ y_bias, TO* __restrict__ out, int R) {
+                                 const float* __restrict__ y_bias, int R) {
   const long total = T * R;
   for (long e = blockIdx.x * (long)blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
     const long t = e / R;
@@ -252,17 +253,17 @@ __global__ void lru_gates_kernel(const float* __restrict__ u, float* __restrict_
     const float la = -8.0f * r * mx_softplus(lam[c]);             // log a
     zp[0] = expf(la);
     zp[bsz] = sqrtf(-expm1f(2.0f * la)) * i * u[e];               // 1 - a^2 without cancellation
-    stf(out + e, gelu_tanh_f(ldf(y + t * sy + c) + (y_bias != nullptr ? y_bias[c] : 0.f)));
+    u[e] = gelu_tanh_f(ldf(y + t * sy + c) + (y_bias != nullptr ? y_bias[c] : 0.f));
   }
 }
 
 constexpr int LRU_CL = 16;      // tokens per thread
 constexpr int LRU_NC = 4;       // thread chunks per block iteration (256 threads: 64 channels x 4)
 
-// grid (ceil(R / 64), S).  z holds a | input term (lru_gates_kernel), out holds the GeLU branch.
+// grid (ceil(R / 64), S).  z holds a | input term, gy the GeLU branch (lru_gates_kernel).
 template <typename TO>
 __global__ void __launch_bounds__(256)
-lru_scan_kernel(const float* __restrict__ z, int bsz, long T, float* __restrict__ state, const int* __restrict__ cu,
+lru_scan_kernel(const float* __restrict__ z, const float* __restrict__ gy, int bsz, long T, float* __restrict__ state, const int* __restrict__ cu,
                 const int* __restrict__ slot, const int* __restrict__ pos, TO* __restrict__ out, int R) {
   __shared__ float sA[LRU_NC][64], sB[LRU_NC][64], sS[64];
   const int s = blockIdx.y;
@@ -285,7 +286,7 @@ lru_scan_kernel(const float* __restrict__ z, int bsz, long T, float* __restrict_
       const long t = r0 + min(first + i, n - 1);
       A[i] = zb[t * 2 * bsz];
       L[i] = zb[t * 2 * bsz + bsz];
-      Gy[i] = ldf(out + t * R + c);
+      Gy[i] = gy[t * R + c];
     }
     float Pp = 1.f, Ll = 0.f;
 #pragma unroll
@@ -385,9 +386,9 @@ MX_API int mx_matrix_scan(const void* q, long sq, const void* k, long sk, const 
                                       slot, pos, out, S, T, H, G, D, P, one, st);
 }
 
-// u f32 [T, R]; z f32 [blocks, T, 2 * R / blocks], OVERWRITTEN with the gates; y [T, >= R] slice (row stride
+// u f32 [T, R], OVERWRITTEN with the GeLU branch; z f32 [blocks, T, 2 * R / blocks], OVERWRITTEN with the gates; y [T, >= R] slice (row stride
 // sy, type dt_y); state f32 [slots, R]; out [T, R] of type dt_out
-MX_API int mx_lru_scan(const float* u, float* z, int blocks, const float* r_bias, const float* i_bias,
+MX_API int mx_lru_scan(float* u, float* z, int blocks, const float* r_bias, const float* i_bias,
                        const float* lam, const void* y, long sy, int dt_y, const float* y_bias, float* state,
                        const int* cu, const int* slot, const int* pos, void* out, int dt_out, int S, int R, int T,
                        hipStream_t st) {
@@ -395,9 +396,9 @@ MX_API int mx_lru_scan(const float* u, float* z, int blocks, const float* r_bias
   if (blocks < 1 || R % blocks) return (int)hipErrorInvalidValue;
   const long total = (long)T * R;
   const int gb = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
-  MX_DISPATCH(dt_y, TY, MX_DISPATCH(dt_out, TO, lru_gates_kernel<TY, TO><<<gb, 256, 0, st>>>(
-      u, z, R / blocks, (long)T, r_bias, i_bias, lam, (const TY*)y, sy, y_bias, (TO*)out, R)));
+  MX_DISPATCH(dt_y, TY, lru_gates_kernel<TY><<<gb, 256, 0, st>>>(u, z, R / blocks, (long)T, r_bias, i_bias, lam, (const TY*)y,
+                                                                 sy, y_bias, R));
   dim3 grid((R + 63) / 64, S);
-  MX_DISPATCH(dt_out, TO, lru_scan_kernel<TO><<<grid, 256, 0, st>>>(z, R / blocks, (long)T, state, cu, slot, pos, (TO*)out, R));
+  MX_DISPATCH(dt_out, TO, lru_scan_kernel<TO><<<grid, 256, 0, st>>>(z, u, R / blocks, (long)T, state, cu, slot, pos, (TO*)out, R));
   MX_RETURN_LAUNCH();
 }

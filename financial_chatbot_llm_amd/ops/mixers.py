@@ -600,7 +600,8 @@ def lru_scan(u: torch.Tensor, z: torch.Tensor, blocks: int, r_bias: torch.Tensor
              slot: torch.Tensor, pos: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     """Per channel, f32: r = sigmoid(zr + r_bias), i = sigmoid(zi + i_bias), a = exp(-8 r softplus(lam)),
     S <- a S + sqrt(1 - a^2) i u (also for a sequence's first token, from S = 0); returns
-    S * gelu_tanh(y + y_bias) in ``out_dtype``.  ``u`` f32 [T, R]; ``z`` f32 [blocks, T, 2 * R / blocks]:
+    S * gelu_tanh(y + y_bias) in ``out_dtype``.  ``u`` f32 [T, R] (the kernels reuse it as scratch);
+    ``z`` f32 [blocks, T, 2 * R / blocks]:
     block b's gate pre-activations [zr | zi] as the batched block-diagonal product leaves them (the
     kernels overwrite it with the gates);
     ``y`` a column slice; ``state`` f32 [slots, R], read unless the segment starts at position 0,
