@@ -85,7 +85,7 @@ def sigudra(width: int) -> int:
         rb, lam = torch.zeros(R, device=dev), torch.zeros(R, device=dev)
         y = torch.randn(T, R, device=dev).bfloat16()
         sl = torch.zeros(S, R, device=dev)
-        us = _time(lambda: mx.lru_scan(uu, z, Bk, rb, rb, lam, y, rb, sl, cu, slot, pos, torch.bfloat16))
+        us = _time(lambda: mx.lru_scan(uu, z, Bk, rb, rb, lam, y, rb, sl, cu, slot, pos, torch.bfloat16, max_len=ml))
         out(shape=name, kernel="lru_scan", us=round(us, 1), TB_per_s=round(T * R * 16 / us / 1e6, 2))
         # windowed attention
         pages = (start + ml + 63) // 64

@@ -21,10 +21,11 @@
 // mx_lru_scan: a diagonal recurrence per channel, S <- a S + sqrt(1 - a^2) i u with
 //     a = exp(-8 sigmoid(zr + r_bias) softplus(lam)),  i = sigmoid(zi + i_bias),
 //   output S * gelu_tanh(y + y_bias).  Two launches: the gates (a, the input term and the GeLU
-//   branch: every transcendental; they replace z and u in place, in f32) elementwise over all rows, then the recurrence itself, where a
-//   block walks 64 tokens at a time: each thread scans 16 tokens of one channel from zero, the four
-//   partial maps S -> A S + B are folded through LDS, and the outputs are corrected by the true
-//   start state.
+//   branch: every transcendental; they replace z and u in place, in f32) elementwise over all rows,
+//   then the recurrence itself, where a block of 16 channels walks 256 tokens at a time: each thread
+//   scans 16 tokens of one channel from zero, the sixteen partial maps S -> A S + B are folded through
+//   LDS, and the outputs are corrected by the true start state.  Steps of single rows (decode) take
+//   one fused launch instead.
 #include "mx_common.h"
 
 namespace {
@@ -258,22 +259,24 @@ __global__ void lru_gates_kernel(float* __restrict__ u, float* __restrict__ z, i
 }
 
 constexpr int LRU_CL = 16;      // tokens per thread
-constexpr int LRU_NC = 4;       // thread chunks per block iteration (256 threads: 64 channels x 4)
+constexpr int LRU_NC = 16;      // thread chunks per block iteration
+constexpr int LRU_CH = 16;      // channels per block (256 threads: 16 channels x 16 chunks, 256 tokens per iteration)
 
-// grid (ceil(R / 64), S).  z holds a | input term, gy the GeLU branch (lru_gates_kernel).
+// grid (ceil(R / LRU_CH), S).  z holds a | input term, gy the GeLU branch (lru_gates_kernel).
 template <typename TO>
 __global__ void __launch_bounds__(256)
-lru_scan_kernel(const float* __restrict__ z, const float* __restrict__ gy, int bsz, long T, float* __restrict__ state, const int* __restrict__ cu,
-                const int* __restrict__ slot, const int* __restrict__ pos, TO* __restrict__ out, int R) {
-  __shared__ float sA[LRU_NC][64], sB[LRU_NC][64], sS[64];
+lru_scan_kernel(const float* __restrict__ z, const float* __restrict__ gy, int bsz, long T, float* __restrict__ state,
+                const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ pos,
+                TO* __restrict__ out, int R) {
+  __shared__ float sA[LRU_NC][LRU_CH], sB[LRU_NC][LRU_CH], sS[LRU_CH];
   const int s = blockIdx.y;
   const int sl = slot[s];
   if (sl < 0) return;
   const int r0 = cu[s], n = cu[s + 1] - r0;
   if (n <= 0) return;
-  const int ch = threadIdx.x & 63, j = threadIdx.x >> 6;
-  const int c = min((int)blockIdx.x * 64 + ch, R - 1);
-  const bool live = (int)blockIdx.x * 64 + ch < R;
+  const int ch = threadIdx.x % LRU_CH, j = threadIdx.x / LRU_CH;
+  const int c = min((int)blockIdx.x * LRU_CH + ch, R - 1);
+  const bool live = (int)blockIdx.x * LRU_CH + ch < R;
   const int b = c / bsz, jj = c - b * bsz;
   const float* zb = z + (long)b * T * 2 * bsz + jj;
   if (j == 0) sS[ch] = pos[r0] == 0 ? 0.f : state[(long)sl * R + c];
@@ -281,12 +284,14 @@ lru_scan_kernel(const float* __restrict__ z, const float* __restrict__ gy, int b
     const int first = t0 + j * LRU_CL;
     const int cnt = max(0, min(LRU_CL, n - first));
     float A[LRU_CL], L[LRU_CL], Gy[LRU_CL];
+    if (cnt > 0) {
 #pragma unroll
-    for (int i = 0; i < LRU_CL; ++i) {          // independent loads, issued together
-      const long t = r0 + min(first + i, n - 1);
-      A[i] = zb[t * 2 * bsz];
-      L[i] = zb[t * 2 * bsz + bsz];
-      Gy[i] = gy[t * R + c];
+      for (int i = 0; i < LRU_CL; ++i) {          // independent loads, issued together
+        const long t = r0 + min(first + i, n - 1);
+        A[i] = zb[t * 2 * bsz];
+        L[i] = zb[t * 2 * bsz + bsz];
+        Gy[i] = gy[t * R + c];
+      }
     }
     float Pp = 1.f, Ll = 0.f;
 #pragma unroll
@@ -311,6 +316,32 @@ lru_scan_kernel(const float* __restrict__ z, const float* __restrict__ gy, int b
     __syncthreads();
   }
   if (j == 0 && live) state[(long)sl * R + c] = sS[ch];
+}
+
+// steps of single rows (decode): gates, recurrence and output in one launch, one thread per (row, channel)
+template <typename TY, typename TO>
+__global__ void lru_step_kernel(const float* __restrict__ u, const float* __restrict__ z, int bsz, long T,
+                                const float* __restrict__ r_bias, const float* __restrict__ i_bias,
+                                const float* __restrict__ lam, const TY* __restrict__ y, long sy,
+                                const float* __restrict__ y_bias, float* __restrict__ state, const int* __restrict__ cu,
+                                const int* __restrict__ slot, const int* __restrict__ pos, TO* __restrict__ out, int S,
+                                int R) {
+  const long total = (long)S * R;
+  for (long e = blockIdx.x * (long)blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
+    const int s = (int)(e / R), c = (int)(e - (long)s * R);
+    const int sl = slot[s];
+    const long t = cu[s];
+    if (sl < 0 || cu[s + 1] <= t) continue;
+    const int b = c / bsz, j = c - b * bsz;
+    const float* zp = z + ((long)b * T + t) * 2 * bsz + j;
+    const float r = mx_sigmoid(zp[0] + r_bias[c]);
+    const float i = mx_sigmoid(zp[bsz] + i_bias[c]);
+    const float la = -8.0f * r * mx_softplus(lam[c]);
+    const float prev = pos[t] == 0 ? 0.f : state[(long)sl * R + c];
+    const float Sn = expf(la) * prev + sqrtf(-expm1f(2.0f * la)) * i * u[t * R + c];
+    state[(long)sl * R + c] = Sn;
+    stf(out + t * R + c, Sn * gelu_tanh_f(ldf(y + t * sy + c) + (y_bias != nullptr ? y_bias[c] : 0.f)));
+  }
 }
 
 template <typename TQ, int RPL, int LPC, bool DELTA>
@@ -345,12 +376,16 @@ template <typename TQ, bool DELTA>
 int run_matrix_scan(const void* q, long sq, const void* k, long sk, const void* v, long sv, float* a, long sa,
                     const float* a_bias, const float* A_log, const void* beta, long sbeta, int beta_dt, float tau_inv,
                     float* aux, float* state, const int* cu, const int* slot, const int* pos, float* out, int S, int T,
-                    int H, int G, int D, int P, bool one, hipStream_t st) {
+                    int H, int G, int D, int P, int max_len, hipStream_t st) {
+  const bool one = max_len == 1;         // every segment is a single row: no chunk staging
   if (!one)        // single-row steps fold this pass into the scan (one launch less per layer)
     scan_prep_kernel<TQ, DELTA><<<T, 256, 0, st>>>((const TQ*)q, sq, (const TQ*)k, sk, a, sa, a_bias, A_log, beta, sbeta,
                                                    beta_dt, tau_inv, aux, H, G, D);
+  // the longest segment sets the step's duration: count the segments that can be about that long (a
+  // prompt chunk beside many single decode rows is still one long chain)
+  const long seff = max_len > 0 ? (S < (T + max_len - 1) / max_len ? S : (T + max_len - 1) / max_len) : S;
   const int lpc = D <= 128 ? 4 : (D <= 256 ? 8 : 16);
-  const long blocks = (long)S * H * ((P + 256 / lpc - 1) / (256 / lpc));
+  const long blocks = seff * H * ((P + 256 / lpc - 1) / (256 / lpc));
   return dispatch_matrix_scan<TQ, DELTA>(D, blocks < 512, q, sq, k, sk, v, sv, (const float*)a, sa, (const float*)aux, state,
                                          cu, slot, pos, out, S, H, G, D, P, a_bias, A_log, beta, sbeta, beta_dt, tau_inv,
                                          one, st);
@@ -368,22 +403,21 @@ MX_API int mx_matrix_scan(const void* q, long sq, const void* k, long sk, const 
                           float tau, int delta, float* aux, float* state, const int* cu, const int* slot, const int* pos,
                           float* out, int S, int T, int max_len, int H, int G, int D, int P, hipStream_t st) {
   if (S <= 0 || T <= 0) return 0;
-  const bool one = max_len == 1;         // every segment is a single row: no chunk staging
   if (D < 1 || D > 512 || G < 1 || H % G || tau <= 0.f || (delta && (A_log == nullptr || beta == nullptr || aux == nullptr)))
     return (int)hipErrorInvalidValue;
   const float ti = 1.0f / tau;
   if (delta) {
     if (dt == 1)
       return run_matrix_scan<float, true>(q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, ti, aux, state,
-                                          cu, slot, pos, out, S, T, H, G, D, P, one, st);
+                                          cu, slot, pos, out, S, T, H, G, D, P, max_len, st);
     return run_matrix_scan<bf16, true>(q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, ti, aux, state, cu,
-                                       slot, pos, out, S, T, H, G, D, P, one, st);
+                                       slot, pos, out, S, T, H, G, D, P, max_len, st);
   }
   if (dt == 1)
     return run_matrix_scan<float, false>(q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, ti, aux, state,
-                                         cu, slot, pos, out, S, T, H, G, D, P, one, st);
+                                         cu, slot, pos, out, S, T, H, G, D, P, max_len, st);
   return run_matrix_scan<bf16, false>(q, sq, k, sk, v, sv, a, sa, a_bias, A_log, beta, sbeta, beta_dt, ti, aux, state, cu,
-                                      slot, pos, out, S, T, H, G, D, P, one, st);
+                                      slot, pos, out, S, T, H, G, D, P, max_len, st);
 }
 
 // u f32 [T, R], OVERWRITTEN with the GeLU branch; z f32 [blocks, T, 2 * R / blocks], OVERWRITTEN with the gates; y [T, >= R] slice (row stride
@@ -391,14 +425,21 @@ MX_API int mx_matrix_scan(const void* q, long sq, const void* k, long sk, const 
 MX_API int mx_lru_scan(float* u, float* z, int blocks, const float* r_bias, const float* i_bias,
                        const float* lam, const void* y, long sy, int dt_y, const float* y_bias, float* state,
                        const int* cu, const int* slot, const int* pos, void* out, int dt_out, int S, int R, int T,
-                       hipStream_t st) {
+                       int max_len, hipStream_t st) {
   if (S <= 0 || T <= 0) return 0;
   if (blocks < 1 || R % blocks) return (int)hipErrorInvalidValue;
+  if (max_len == 1) {
+    const long tot = (long)S * R;
+    const int g1 = (int)((tot + 255) / 256 < 8192 ? (tot + 255) / 256 : 8192);
+    MX_DISPATCH(dt_y, TY, MX_DISPATCH(dt_out, TO, lru_step_kernel<TY, TO><<<g1, 256, 0, st>>>(
+        u, z, R / blocks, (long)T, r_bias, i_bias, lam, (const TY*)y, sy, y_bias, state, cu, slot, pos, (TO*)out, S, R)));
+    MX_RETURN_LAUNCH();
+  }
   const long total = (long)T * R;
   const int gb = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
   MX_DISPATCH(dt_y, TY, lru_gates_kernel<TY><<<gb, 256, 0, st>>>(u, z, R / blocks, (long)T, r_bias, i_bias, lam, (const TY*)y,
                                                                  sy, y_bias, R));
-  dim3 grid((R + 63) / 64, S);
+  dim3 grid((R + LRU_CH - 1) / LRU_CH, S);
   MX_DISPATCH(dt_out, TO, lru_scan_kernel<TO><<<grid, 256, 0, st>>>(z, u, R / blocks, (long)T, state, cu, slot, pos, (TO*)out, R));
   MX_RETURN_LAUNCH();
 }

@@ -528,7 +528,7 @@ class GatedLRUMixer:
                         meta.seg_max_len, "none", in_bias=self.x_b)
         z = torch.bmm(u.view(T, B, bs).transpose(0, 1), self.w_ri)             # [B, T, 2 bs]: r | i pre-activations
         s = mx.lru_scan(u, z, B, self.r_b, self.i_b, self.lam, proj[:, :R], self.y_b, st["S"], meta.seg_cu,
-                        meta.seg_state, positions, proj.dtype)
+                        meta.seg_state, positions, proj.dtype, max_len=meta.seg_max_len)
         return F.linear(s, self.o)
 
 

@@ -101,7 +101,7 @@ _MIXER_SIGS = {
     "mx_head_norm_gate": [P, c_long, c_int, P, c_float, P, c_long, c_int, c_int, P, c_int, c_int, c_int, c_int, P],
     "mx_matrix_scan": [P, c_long, P, c_long, P, c_long, c_int, P, c_long, P, P, P, c_long, c_int, c_float, c_int, P, P, P, P,
                        P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
-    "mx_lru_scan": [P, P, c_int, P, P, P, P, c_long, c_int, P, P, P, P, P, P, c_int, c_int, c_int, c_int, P],
+    "mx_lru_scan": [P, P, c_int, P, P, P, P, c_long, c_int, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mx_qk_norm_write": [P, c_long, P, c_long, P, c_long, P, P, c_float, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mx_window_attend": [P, c_long, P, P, P, P, c_int, P, c_long, c_int, c_float, P, c_int, c_int, c_int, c_int, c_int,
                          c_int, c_int, c_int, P, P],

@@ -597,7 +597,7 @@ def head_norm_gate(o: torch.Tensor, w: torch.Tensor, eps: float, gate: torch.Ten
 # ----------------------------------------------------------------------------------------------
 def lru_scan(u: torch.Tensor, z: torch.Tensor, blocks: int, r_bias: torch.Tensor, i_bias: torch.Tensor,
              lam: torch.Tensor, y: torch.Tensor, y_bias: Optional[torch.Tensor], state: torch.Tensor, cu: torch.Tensor,
-             slot: torch.Tensor, pos: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+             slot: torch.Tensor, pos: torch.Tensor, out_dtype: torch.dtype, max_len: int = 0) -> torch.Tensor:
     """Per channel, f32: r = sigmoid(zr + r_bias), i = sigmoid(zi + i_bias), a = exp(-8 r softplus(lam)),
     S <- a S + sqrt(1 - a^2) i u (also for a sequence's first token, from S = 0); returns
     S * gelu_tanh(y + y_bias) in ``out_dtype``.  ``u`` f32 [T, R] (the kernels reuse it as scratch);
@@ -605,7 +605,7 @@ def lru_scan(u: torch.Tensor, z: torch.Tensor, blocks: int, r_bias: torch.Tensor
     block b's gate pre-activations [zr | zi] as the batched block-diagonal product leaves them (the
     kernels overwrite it with the gates);
     ``y`` a column slice; ``state`` f32 [slots, R], read unless the segment starts at position 0,
-    then replaced."""
+    then replaced.  ``max_len``: the longest segment when known (1 selects the fused single-row kernel)."""
     T, R = u.shape
     S = cu.numel() - 1
     bs = R // blocks
@@ -615,7 +615,7 @@ def lru_scan(u: torch.Tensor, z: torch.Tensor, blocks: int, r_bias: torch.Tensor
         out = torch.empty((T, R), dtype=out_dtype, device=u.device)
         N.mcall("mx_lru_scan", N.ptr(u), N.ptr(z), blocks, N.ptr(r_bias), N.ptr(i_bias), N.ptr(lam), N.ptr(_rows(y)),
                 y.stride(0), _dt(y), N.ptr(y_bias), N.ptr(state), N.ptr(cu), N.ptr(slot), N.ptr(pos), N.ptr(out), _dt(out),
-                S, R, T, N.stream())
+                S, R, T, int(max_len), N.stream())
         return out
     zr = z[:, :, :bs].transpose(0, 1).reshape(T, R)
     zi = z[:, :, bs:].transpose(0, 1).reshape(T, R)
