@@ -319,12 +319,15 @@ class InputScaledRoutedFF:
         offs = [0] + torch.bincount(flat, minlength=E).cumsum(0).tolist()              # host read of the buckets
         xs = h.index_select(0, order // top)
         sc = wts.reshape(-1)[order].contiguous()
+        # one GEMM pair per expert with rows; the activation runs once over all buckets
+        gu = torch.empty((T * top, 2 * Fe), dtype=h.dtype, device=h.device)
+        live = [(e, offs[e], offs[e + 1]) for e in range(E) if offs[e + 1] > offs[e]]
+        for e, a, b in live:
+            torch.mm(xs[a:b], self.w13[e].t(), out=gu[a:b])
+        act = mx.glu_act(gu[:, :Fe], gu[:, Fe:], self.act, sc)
         ys = torch.empty((T * top, W), dtype=h.dtype, device=h.device)
-        for e in range(E):
-            a, b = offs[e], offs[e + 1]
-            if b > a:
-                gu = F.linear(xs[a:b], self.w13[e])
-                torch.mm(mx.glu_act(gu[:, :Fe], gu[:, Fe:], self.act, sc[a:b]), self.w2[e].t(), out=ys[a:b])
+        for e, a, b in live:
+            torch.mm(act[a:b], self.w2[e].t(), out=ys[a:b])
         pos = torch.empty_like(order)
         pos[order] = torch.arange(order.numel(), device=order.device)
         return mx.moe_combine(ys, pos.view(T, top).to(torch.int32), idx, ones, h, None, E)
