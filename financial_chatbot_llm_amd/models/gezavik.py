@@ -58,7 +58,7 @@ def example_config(width: int = 192, vocab: int = 1024, heads: int = 3, pattern:
 
 class _Layer(Layer):
     def __init__(self, i: int, spec: Dict, width: int, eps: float):
-        super().__init__(i, spec, width, eps)
+        super().__init__(i, spec, width, eps, GezavikModel.mixer_types)
         mlp = spec.get("mlp")
         if mlp is None:
             self.ff = None

@@ -21,7 +21,8 @@ from .mixers import MIXERS
 
 
 class Layer:
-    """One layer: its mixer, its feed-forward (``ff``, set by the design) and its loaded norms."""
+    """One layer: its mixer (one of the design's ``mixer_types``), its feed-forward (``ff``, set by the
+    design) and its loaded norms."""
     norm_names = ("norm1",)
 
     def __init__(self, i: int, spec: Dict, width: int, eps: float, mixer_types=None):
