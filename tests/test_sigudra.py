@@ -401,6 +401,41 @@ def test_lru_state_carries_far(device):
         assert (out[:2] == 0).all()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("lens", [[15, 16, 17, 33], [255, 257], [600, 1, 300]])
+def test_segments_across_the_kernels_chunks(lens):
+    """Segments whose lengths sit on and around the kernels' internal chunk sizes (16 tokens of the matrix
+    scan, 16 x 16 tokens of the LRU fold), several per step, against the ops' plain forms on the CPU."""
+    g = torch.Generator().manual_seed(sum(lens))
+    T, S = sum(lens), len(lens)
+    cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32)
+    pos = torch.cat([torch.arange(7 * i, 7 * i + n) for i, n in enumerate(lens)]).to(torch.int32)   # the first starts at 0
+    slot = torch.arange(S, dtype=torch.int32).flip(0)
+    dev = lambda *ts: [t.cuda() for t in ts]  # noqa: E731
+    H, G, D, P = 3, 1, 40, 24
+    for mode in ("gla", "delta"):
+        q, k, v = torch.randn(T, G * D, generator=g), torch.randn(T, G * D, generator=g) * 0.2, torch.randn(T, H * P, generator=g)
+        a = torch.randn(T, H * D, generator=g) + 3
+        ab, Al, beta = torch.zeros(H * D), torch.zeros(H), torch.randn(T, H, generator=g)
+        st = torch.randn(S, H, D, P, generator=g) * 0.1
+        s1, s2 = st.clone(), st.clone().cuda()
+        want = mx.matrix_scan(q, k, v, a.clone(), ab, s1, cu, slot, pos, H, G, D, P, mode, tau=4.0, A_log=Al, beta=beta)
+        got = mx.matrix_scan(*dev(q, k, v, a.clone(), ab), s2, *dev(cu, slot, pos), H, G, D, P, mode, tau=4.0, A_log=Al.cuda(),
+                             beta=beta.cuda(), max_len=max(lens))
+        assert (got.cpu() - want).abs().max() <= 2e-4 * want.abs().max()
+        assert (s2.cpu() - s1).abs().max() <= 2e-4 * s1.abs().max()
+    R, Bk = 40, 2
+    u, z = torch.randn(T, R, generator=g), torch.randn(Bk, T, 2 * R // Bk, generator=g)
+    rb, ib, lam, y = torch.zeros(R), torch.zeros(R), torch.randn(R, generator=g) - 2, torch.randn(T, R, generator=g)
+    st = torch.randn(S, R, generator=g)
+    s1, s2 = st.clone(), st.clone().cuda()
+    want = mx.lru_scan(u.clone(), z.clone(), Bk, rb, ib, lam, y, None, s1, cu, slot, pos, torch.float32)
+    got = mx.lru_scan(*dev(u.clone(), z.clone()), Bk, *dev(rb, ib, lam, y), None, s2, *dev(cu, slot, pos), torch.float32,
+                      max_len=max(lens))
+    assert (got.cpu() - want).abs().max() <= 2e-5 * want.abs().max()
+    assert (s2.cpu() - s1).abs().max() <= 2e-5 * s1.abs().max().clamp(min=1.0)
+
+
 # ---------------------------------------------------------------------------------------------------
 # routing, embedding
 # ---------------------------------------------------------------------------------------------------
